@@ -1,0 +1,147 @@
+/* C ABI of libtriteia_hip.so -- the MI355X (gfx950) implementation of Triteia's
+ * fp16 x (int4, 2:4-sparse) multi-model GEMM path and its LoRA companions.
+ *
+ * Every entry point takes plain device pointers and sizes, enqueues its work on
+ * `stream` (a hipStream_t passed as void*; NULL = the default stream) of
+ * device `dev`, and returns without synchronising.  Nothing is allocated or
+ * freed by the library; all buffers, including workspaces, belong to the
+ * caller and are borrowed until the enqueued work has run.
+ *
+ * Dimension names follow the reference launchers: prob_m = output features,
+ * prob_n = tokens (rows of A / C), prob_k = input features.
+ *
+ * Tensor layouts (identical to the reference's, see its packer
+ * triteia/python/nn/linear.py:79-141):
+ *   A     fp16  [prob_n, prob_k]            row-major activations
+ *   B     int32 [prob_k/32, 2*prob_m]       packed 2:4 int4 weights
+ *   meta  int16 [prob_m, prob_k/16]         2:4 metadata (Sparse-Marlin order)
+ *   s     fp16  [1, prob_m]                 per-output-channel scales
+ *   C     fp16  [prob_n, prob_m]            row-major output
+ * Batched variants carry a leading delta dimension on B / meta / s.
+ *
+ * Return codes: 0 on success, otherwise one of the TRITEIA_HIP_ERR_* values;
+ * triteia_hip_last_error() describes the last failure on the calling thread.
+ */
+#ifndef TRITEIA_HIP_H_
+#define TRITEIA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define TRITEIA_HIP_API __attribute__((visibility("default")))
+#else
+#define TRITEIA_HIP_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRITEIA_HIP_OK 0
+#define TRITEIA_HIP_ERR_PROB_SHAPE 1 /* reference: ERR_PROB_SHAPE, csrc/ops/marlin_nm.cu:39 */
+#define TRITEIA_HIP_ERR_KERN_SHAPE 2 /* reference: ERR_KERN_SHAPE, csrc/ops/marlin_nm.cu:40 */
+#define TRITEIA_HIP_ERR_ARGUMENT 3   /* null pointer, undersized workspace, bad flag */
+#define TRITEIA_HIP_ERR_RUNTIME 4    /* a HIP call failed */
+
+/* Library / ABI version (major * 1000 + minor). */
+TRITEIA_HIP_API int triteia_hip_version(void);
+
+/* Text of the last error raised on this thread ("" if none). */
+TRITEIA_HIP_API const char* triteia_hip_last_error(void);
+
+/* C = A @ dequant(B, meta, s) for one weight matrix.
+ * Replaces marlin_cuda_2_4 (triteia/csrc/ops/marlin_nm.cu:42-46), bound by the
+ * reference as mul_2_4 (triteia/csrc/ops/ops.cpp:88-116).
+ * workspace: the reference's lock array (>= prob_m/128*max_par int32 zeros); it
+ * is accepted, never read or written, and therefore left all-zero.
+ * groupsize must be -1 (per-channel scales).  thread_k, thread_m, sms, max_par
+ * are the reference's tuning knobs; they are accepted and ignored.
+ * Shape rules: prob_m % 128 == 0 and prob_k % 64 == 0, else ERR_PROB_SHAPE. */
+TRITEIA_HIP_API int triteia_hip_mul_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m, int prob_n,
+                        int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k, int thread_m,
+                        int sms, int max_par);
+
+/* C[b, 0, :] = A[b, 0, :] @ dequant(B[b]) for b < prob_n: one token per matrix.
+ * Replaces triteia_cuda_bmm_2_4 (triteia/csrc/ops/triteia_nm_bmm.cu:760-764),
+ * bound as bmm_2_4 (triteia/csrc/ops/ops.cpp:240-277).  prob_n = batch. */
+TRITEIA_HIP_API int triteia_hip_bmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m, int prob_n,
+                        int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k, int thread_m,
+                        int sms, int max_par);
+
+/* Same with `tokens` rows per matrix: A [batch, tokens, k], C [batch, tokens, m].
+ * The reference kernel hard-codes tokens == 1 (triteia_nm_bmm.cu:736-739); its
+ * Python for-loop variant (triteia/python/ops/matmul/bmm.py:6-18) defines the
+ * semantics for tokens > 1. */
+TRITEIA_HIP_API int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
+                               int batch, int tokens, int prob_k, int dev, void* stream);
+
+/* Run-list form: for run r < prob_r, rows starts[r] .. starts[r]+counts[r]-1 of
+ * C = same rows of A @ dequant(B[indices[r]]).  indices / starts / counts are
+ * int32 device arrays.  Replaces triteia_cuda_sbmm_2_4
+ * (triteia/csrc/ops/triteia_nm_sbmm.cu:809-815), bound as sbmm_2_4 and, for the
+ * host-loop variant, sbmm_forloop (triteia/csrc/ops/ops.cpp:279-327).
+ * Rows not covered by a run are left untouched; runs with indices[r] outside
+ * [0, n_deltas) are skipped.  n_deltas = number of matrices in B. */
+TRITEIA_HIP_API int triteia_hip_sbmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, const void* indices,
+                         const void* starts, const void* counts, int prob_m, int prob_n, int prob_k, int prob_r,
+                         int n_deltas, void* workspace, int groupsize, int dev, void* stream, int thread_k,
+                         int thread_m, int sms, int max_par);
+
+/* Per-token routed form (no counterpart kernel in the reference; it replaces the
+ * host-side routing prep of triteia/python/ops/matmul/sbmm.py:94-123 plus the
+ * kernel above plus the trailing `y += output`, sbmm.py:141):
+ *   d = token_indices[t] - index_offset
+ *   0 <= d < n_deltas :  C[t] = (accumulate ? C[t] : 0) + A[t] @ dequant(B[d])
+ *   otherwise         :  C[t] untouched
+ * token_indices: int32 [prob_n] on the device, any order.  The tokens are
+ * grouped on the device, so each delta's weights are read once per launch.
+ * workspace: >= triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas) bytes
+ * of device memory, contents irrelevant on entry, overwritten.
+ * n_deltas <= 8192. */
+TRITEIA_HIP_API int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                const void* token_indices, int index_offset, int n_deltas, int prob_m, int prob_n,
+                                int prob_k, void* workspace, size_t workspace_bytes, int accumulate, int dev,
+                                void* stream);
+TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n_deltas);
+
+/* Only the routing step of the call above: fills `workspace` with
+ * [n_groups, n_routed, 0, 0 | g_delta[G] | g_start[G] | g_count[G] | perm[prob_n]]
+ * (int32, G = min(prob_n, n_deltas)).  Exposed so that the LoRA path can share
+ * one routing pass with the delta path. */
+TRITEIA_HIP_API int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
+                           size_t workspace_bytes, int dev, void* stream);
+
+/* BGMV: Y[b, :] += scale * W[indices[b] * num_layers + layer_idx] @ X[b, :]
+ * with W [n, num_layers, h_out, h_in] fp16 (out-major) and indices int64 [batch]
+ * (negative = skip).  Replaces bgmv_kernel<feat_in, feat_out, T>
+ * (triteia/csrc/ops/bgmv_config.h:3-7, bgmv_impl.cuh:185-207), bound as
+ * dispatch_bgmv (triteia/csrc/ops/ops.cpp:177-220).  Unlike the reference it
+ * runs on `stream`, and shapes are run-time values: both sides multiples of 8
+ * and min(h_in, h_out) <= 128, else ERR_KERN_SHAPE ("No suitable kernel"). */
+TRITEIA_HIP_API int triteia_hip_bgmv(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                     int num_layers, int layer_idx, float scale, int dev, void* stream);
+
+/* SGMV: y[s[i] : s[i+1]] += x[s[i] : s[i+1]] @ W_i, W_i = (fp16*)w_ptrs[i] +
+ * layer_idx * d_in * d_out, row-major [d_in, d_out]; s int32 [num_problems+1].
+ * Replaces sgmv<T> (triteia/csrc/ops/sgmv.h:6-11, sgmv.cuh:61-174), bound as
+ * dispatch_sgmv_cutlass (triteia/csrc/ops/ops.cpp:120-147).  tmp is the
+ * reference's CUTLASS argument scratch; it is accepted and unused. */
+TRITEIA_HIP_API int triteia_hip_sgmv(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
+                     int d_out, int layer_idx, int dev, void* stream);
+TRITEIA_HIP_API size_t triteia_hip_sgmv_tmp_size(int num_problems); /* reference: sgmv_tmp_size, sgmv.cuh:48-52 */
+
+/* Routed SGMV on a routing plan made by triteia_hip_route_plan: for every group
+ * g (adapter a = g_delta[g]) and every listed row t:
+ *   y[t] += scale * x[t] @ W[a],  W = w_base + a * w_stride (elements),
+ *   row-major [d_in, d_out].
+ * No counterpart in the reference, which builds the segment table on the host
+ * (triteia/python/ops/matmul/lora.py:63-96). */
+TRITEIA_HIP_API int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
+                            int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
+                            int dev, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRITEIA_HIP_H_ */

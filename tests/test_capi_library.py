@@ -1,0 +1,76 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every declared symbol, and rejects
+bad problems before touching the GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from triteia_amd.python.capi import _ffi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "triteia_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(triteia_hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_symbols()
+    assert len(names) >= 12
+    handle = ctypes.CDLL(_ffi.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), f"{n} declared in include/triteia_hip.h but not exported"
+    assert set(names) == set(_ffi.SIGNATURES), "ctypes table and header disagree"
+
+
+def test_version_and_error_text():
+    lib = _ffi.lib()
+    assert lib.triteia_hip_version() >= 1000
+    assert isinstance(_ffi.last_error(), str)
+
+
+@pytest.mark.parametrize("m,n,k,gs,code", [
+    (100, 16, 4096, -1, _ffi.ERR_PROB_SHAPE),      # m not a multiple of 128
+    (4096, 16, 100, -1, _ffi.ERR_PROB_SHAPE),      # k not a multiple of 64
+    (4096, 16, 4096, 64, _ffi.ERR_KERN_SHAPE),     # grouped scales are not implemented
+    (4096, 0, 4096, -1, 0),                        # empty problem is a no-op
+])
+def test_shape_errors_do_not_need_a_gpu(m, n, k, gs, code):
+    lib = _ffi.lib()
+    null = ctypes.c_void_p(0)
+    rc = lib.triteia_hip_mul_2_4(null, null, null, null, null, m, n, k, null, gs, 0, null, -1, -1, -1, 16)
+    assert rc == code
+    if code:
+        assert _ffi.last_error() != ""
+    rc = lib.triteia_hip_bmm_2_4(null, null, null, null, null, m, n, k, null, gs, 0, null, -1, -1, -1, 16)
+    assert rc == code
+
+
+def test_other_argument_errors():
+    lib = _ffi.lib()
+    null = ctypes.c_void_p(0)
+    # bgmv: narrow side too wide / not a multiple of 8
+    assert lib.triteia_hip_bgmv(null, null, null, null, 4, 4096, 256, 1, 0, 1.0, 0, null) == _ffi.ERR_KERN_SHAPE
+    assert "No suitable kernel" in _ffi.last_error()
+    assert lib.triteia_hip_bgmv(null, null, null, null, 4, 4096, 12, 1, 0, 1.0, 0, null) == _ffi.ERR_KERN_SHAPE
+    assert lib.triteia_hip_bgmv(null, null, null, null, 4, 4096, 16, 1, 3, 1.0, 0, null) == _ffi.ERR_PROB_SHAPE
+    # routed sbmm: workspace too small, too many deltas
+    need = lib.triteia_hip_sbmm_routed_workspace_bytes(64, 16)
+    assert need == 4 * (4 + 3 * 16 + 64)
+    one = ctypes.c_void_p(1)
+    assert lib.triteia_hip_route_plan(one, 0, 16, 64, one, need - 1, 0, null) == _ffi.ERR_ARGUMENT
+    assert lib.triteia_hip_route_plan(one, 0, 100000, 64, one, 1 << 30, 0, null) == _ffi.ERR_KERN_SHAPE
+    assert lib.triteia_hip_sgmv_tmp_size(7) == 420
+    assert lib.triteia_hip_sgmv(null, null, null, null, null, 0, 4096, 16, 0, 0, null) == 0
+
+
+def test_python_wrappers_refuse_cpu_tensors():
+    import torch
+    from triteia_amd.python.ops import matmul_4bit_2_4
+    x = torch.zeros(2, 128, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        matmul_4bit_2_4(torch.zeros(4, 512, dtype=torch.int32), x, torch.zeros(256, 8, dtype=torch.int16),
+                        torch.ones(1, 256, dtype=torch.float16))

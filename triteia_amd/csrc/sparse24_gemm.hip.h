@@ -1,0 +1,294 @@
+// fp16 x (int4, 2:4-sparse) grouped GEMM for gfx950 (MI355X).
+//
+// One kernel serves matmul_4bit_2_4, bmm_4bit_2_4 and the routed
+// sbmm_4bit_2_4 / ldmm delta path: the work is a list of *groups*, each group
+// being (delta matrix, list of token rows).  A workgroup owns one
+// (group, 128-output-column block) and streams that slice of the packed
+// weights from HBM exactly once per 16*NT tokens.
+//
+// Packed layout consumed directly (no repacking), as produced by the
+// reference's packer (triteia/python/nn/linear.py:79-141,
+// triteia/python/ops/utils/sparsity.py:35-61,134-161):
+//   qweight [k/32][2m] int32 : per 32-dense-k row `tr`, 64 output columns are
+//       128 consecutive int32 = 32 x 16-byte vectors.  Vector i holds output
+//       columns 8*(i/4)..+7 and compressed-k entries {2a,2a+1,2a+8,2a+9},
+//       a = i%4, i.e. 2:4 groups a and a+4 of the 8 groups in the row.
+//   meta [k/32][m][2] int16 (physical order): per `tr`, 64 columns are 128
+//       int16 whose index has bits [b1 b5 b4 b3 b0 h b2] (b = column bits,
+//       h = which 16-k half); each int16 = four 4-bit (lo | hi<<2) codes.
+//   scales [m] fp16 per output column.
+//
+// Mapping onto V_SMFMAC_F32_16X16X64_F16 (sparse A = weights, dense B =
+// activations, D = out^T tile):
+//   lane l = (r = l%16, q = l/16).  Row r of the MFMA is the 8-column block r
+//   of the 128-column block; quarter q covers packed row tr0+q.  For output
+//   column c (0..7) inside the block and k-half u (0/1) one MFMA consumes, per
+//   lane, the 4 groups {4u..4u+3} of that column: one half2 from each of the
+//   lane's four 16-byte weight vectors, and exactly one 16-bit metadata word
+//   as the index operand (ABID selects the half of the 32-bit word).  The
+//   dequantised half2 comes from the (nibble | 0x6400) - 1032 trick, so the
+//   weights go HBM -> VGPR -> MFMA with ~2 VALU ops per pair.
+//   B operand of lane (n = l%16, qb = l/16): 8 halfs from
+//   x[token n][32*(tr0 + qb/2) + 16u + 8*(qb%2) ..] and 8 from the same
+//   offset two packed rows further (the instruction's K order for B is
+//   {8qb..8qb+7, 32+8qb..}).
+//   D: lane (n, qq) holds rows 4qq+j => output features 32qq + 8j + c: 32
+//   consecutive features of token n.
+//
+// The KW wavefronts of a workgroup split K between them and reduce through
+// LDS in a fixed order (deterministic, no atomics, no global scratch).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace triteia_hip {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half16_t __attribute__((ext_vector_type(16)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+struct Sparse24Args {
+  const _Float16* x;        // [T, k] activations
+  long x_stride;            // elements between token rows
+  const uint4_t* qweight;   // [N][k/32][m/2] 16-byte vectors
+  long qweight_stride;      // vectors between deltas
+  const uint4_t* meta;      // [N][k/32][m/4] 16-byte vectors (physical order)
+  long meta_stride;         // vectors between deltas
+  const _Float16* scales;   // [N][m]
+  long scales_stride;       // elements between deltas
+  _Float16* out;            // [T, m]
+  long out_stride;          // elements between rows
+  int m;                    // output features
+  int k;                    // input features
+  // groups: explicit arrays, or (if g_delta == nullptr) group j = delta
+  // j*delta_step with rows [j*uniform_count, (j+1)*uniform_count)
+  const int* g_delta;
+  const int* g_start;
+  const int* g_count;
+  const int* perm;          // row of the i-th listed token (nullptr: identity)
+  const int* n_groups_dev;  // device-side group count (nullptr: n_groups)
+  int n_groups;             // upper bound on the number of groups
+  int uniform_count;
+  int delta_step;
+  int n_deltas;             // deltas with index outside [0, n_deltas) are skipped
+  int accumulate;           // 0: out = result, 1: out += result
+};
+
+__device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ __forceinline__ half2_t bits_h2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
+
+// nibbles 0 and 4 of w -> (n0 - 8, n4 - 8)
+__device__ __forceinline__ uint32_t dequant_even(uint32_t w) {
+  const half2_t bias = {(_Float16)1032.0f, (_Float16)1032.0f};
+  return h2_bits(bits_h2((w & 0x000f000fu) | 0x64006400u) - bias);
+}
+// nibbles 1 and 5 of w -> (n1 - 8, n5 - 8):  (1024 + 16 n) / 16 - 72
+__device__ __forceinline__ uint32_t dequant_odd(uint32_t w) {
+  const half2_t mul = {(_Float16)0.0625f, (_Float16)0.0625f};
+  const half2_t add = {(_Float16)-72.0f, (_Float16)-72.0f};
+  return h2_bits(bits_h2((w & 0x00f000f0u) | 0x64006400u) * mul + add);
+}
+
+template <int NT>
+struct StepFrag {
+  uint4_t wq[4];        // weights: groups a and a+4 (a = vector index) of 8 columns
+  uint4_t mt[2];        // metadata vectors (b1 = 0, 1)
+  uint4_t xa[NT][2];    // B slots 0..7 for u = 0, 1
+  uint4_t xb[NT][2];    // B slots 8..15 for u = 0, 1
+};
+
+constexpr int kRedStride = 132;  // floats per token row in the reduction buffer (128 + pad)
+
+template <int NT, int KW>
+__global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse24Args p) {
+  __shared__ float red[KW][16][kRedStride];
+  __shared__ int s_rows[16 * NT];
+
+  const int col_blocks = p.m >> 7;
+  const int unit = blockIdx.x;
+  const int grp = unit / col_blocks;
+  const int cb = unit - grp * col_blocks;
+  const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
+  if (grp >= n_groups) return;
+
+  int delta, start, count;
+  if (p.g_delta) {
+    delta = p.g_delta[grp];
+    start = p.g_start[grp];
+    count = p.g_count[grp];
+  } else {
+    delta = grp * p.delta_step;
+    start = grp * p.uniform_count;
+    count = p.uniform_count;
+  }
+  if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int r = lane & 15;
+  const int q = lane >> 4;
+
+  const int k_rows = p.k >> 5;                 // packed rows (32 dense k each)
+  const int n_steps = (k_rows + 3) >> 2;       // 128 dense k per step
+  const long qrow = p.m >> 1;                  // vectors per packed weight row
+  const long mrow = p.m >> 2;                  // vectors per packed metadata row
+
+  const uint4_t* qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * r;
+  const uint4_t* mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (r >> 3)) * 16 + (r & 7);
+  const _Float16* sc = p.scales + (long)delta * p.scales_stride + cb * 128;
+
+  // blockIdx.y splits a group's tokens between workgroups (each re-streams the weights)
+  for (int t0 = blockIdx.y * 16 * NT; t0 < count; t0 += gridDim.y * 16 * NT) {
+    const int cnt = min(count - t0, 16 * NT);
+    __syncthreads();  // previous pass finished reading s_rows / red
+    if (tid < 16 * NT) {
+      int row = -1;
+      if (tid < cnt) row = p.perm ? p.perm[start + t0 + tid] : start + t0 + tid;
+      s_rows[tid] = row;
+    }
+    __syncthreads();
+
+    const _Float16* xrow[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const int row = s_rows[nt * 16 + r];
+      // B operand slot layout: this lane supplies k offsets 8*(q%2) + {0..7} of
+      // packed rows tr0 + q/2 and tr0 + 2 + q/2
+      xrow[nt] = row >= 0 ? p.x + (long)row * p.x_stride + 32 * (q >> 1) + 8 * (q & 1) : nullptr;
+    }
+
+    float4_t acc[8][NT];
+#pragma unroll
+    for (int c = 0; c < 8; c++)
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) acc[c][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    auto load_step = [&](StepFrag<NT>& f, int st) {
+      const int tr0 = st << 2;
+      const int tr = min(tr0 + q, k_rows - 1);  // clamped: rows past the end are cancelled by zero B
+      const uint4_t* wp = qw_lane + (long)tr * qrow;
+#pragma unroll
+      for (int a = 0; a < 4; a++) f.wq[a] = __builtin_nontemporal_load(wp + a);
+      const uint4_t* mp = mt_lane + (long)tr * mrow;
+      f.mt[0] = __builtin_nontemporal_load(mp);
+      f.mt[1] = __builtin_nontemporal_load(mp + 8);
+      const bool ok_a = (tr0 + (q >> 1)) < k_rows;
+      const bool ok_b = (tr0 + 2 + (q >> 1)) < k_rows;
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        const uint4_t zero = {0u, 0u, 0u, 0u};
+        f.xa[nt][0] = f.xa[nt][1] = f.xb[nt][0] = f.xb[nt][1] = zero;
+        if (xrow[nt] != nullptr && nt * 16 < cnt) {
+          const _Float16* xp = xrow[nt] + (long)tr0 * 32;
+          if (ok_a) {
+            f.xa[nt][0] = *reinterpret_cast<const uint4_t*>(xp);
+            f.xa[nt][1] = *reinterpret_cast<const uint4_t*>(xp + 16);
+          }
+          if (ok_b) {
+            f.xb[nt][0] = *reinterpret_cast<const uint4_t*>(xp + 64);
+            f.xb[nt][1] = *reinterpret_cast<const uint4_t*>(xp + 80);
+          }
+        }
+      }
+    };
+
+    auto compute_step = [&](const StepFrag<NT>& f) {
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        half16_t b[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+          typedef uint32_t uint8_t_v __attribute__((ext_vector_type(8)));
+          uint8_t_v bb = {f.xa[nt][u][0], f.xa[nt][u][1], f.xa[nt][u][2], f.xa[nt][u][3],
+                          f.xb[nt][u][0], f.xb[nt][u][1], f.xb[nt][u][2], f.xb[nt][u][3]};
+          b[nt] = __builtin_bit_cast(half16_t, bb);
+        }
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+          const int w = c & 3;         // word inside each weight vector
+          const int b2 = c >> 2;       // upper / lower 4 columns of the 8-column block
+          uint4_t av;
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            uint32_t word = f.wq[a][w];
+            if (b2) word >>= 8;
+            av[a] = u ? dequant_odd(word) : dequant_even(word);
+          }
+          const half8_t A = __builtin_bit_cast(half8_t, av);
+          const int idx = (int)f.mt[(c >> 1) & 1][(c & 1) * 2 + u];
+#pragma unroll
+          for (int nt = 0; nt < NT; nt++) {
+            if (nt * 16 < cnt) {
+              if (b2)
+                acc[c][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A, b[nt], acc[c][nt], idx, 0, 1);
+              else
+                acc[c][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A, b[nt], acc[c][nt], idx, 0, 0);
+            }
+          }
+        }
+      }
+    };
+
+    // K loop: wave w takes steps w, w + KW, ...; one step of register prefetch
+    StepFrag<NT> cur, nxt;
+    int st = wave;
+    if (st < n_steps) load_step(cur, st);
+    while (st < n_steps) {
+      const int st_next = st + KW;
+      if (st_next < n_steps) load_step(nxt, st_next);
+      compute_step(cur);
+      cur = nxt;
+      st = st_next;
+    }
+
+    // cross-wave reduction + epilogue, one 16-token tile at a time
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      if (nt * 16 >= cnt) break;
+      if (nt > 0) __syncthreads();
+      float* dst = &red[wave][r][32 * q];   // D: lane (n = r, qq = q) owns features 32q + 8j + c
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float4_t lo = {acc[0][nt][j], acc[1][nt][j], acc[2][nt][j], acc[3][nt][j]};
+        float4_t hi = {acc[4][nt][j], acc[5][nt][j], acc[6][nt][j], acc[7][nt][j]};
+        *reinterpret_cast<float4_t*>(dst + 8 * j) = lo;
+        *reinterpret_cast<float4_t*>(dst + 8 * j + 4) = hi;
+      }
+      __syncthreads();
+      // 16 tokens x 128 features = 256 chunks of 8 features
+      for (int ch = tid; ch < 256; ch += 64 * KW) {
+        const int tok = ch >> 4;
+        const int f0 = (ch & 15) * 8;
+        const int row = s_rows[nt * 16 + tok];
+        if (row < 0) continue;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = 0.f;
+#pragma unroll
+        for (int w = 0; w < KW; w++) {
+          const float4_t a0 = *reinterpret_cast<const float4_t*>(&red[w][tok][f0]);
+          const float4_t a1 = *reinterpret_cast<const float4_t*>(&red[w][tok][f0 + 4]);
+#pragma unroll
+          for (int i = 0; i < 4; i++) { v[i] += a0[i]; v[4 + i] += a1[i]; }
+        }
+        const half8_t sv = *reinterpret_cast<const half8_t*>(sc + f0);
+        _Float16* op = p.out + (long)row * p.out_stride + cb * 128 + f0;
+        half8_t o;
+        if (p.accumulate) {
+          const half8_t old = *reinterpret_cast<const half8_t*>(op);
+#pragma unroll
+          for (int i = 0; i < 8; i++) o[i] = (_Float16)((float)old[i] + v[i] * (float)sv[i]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; i++) o[i] = (_Float16)(v[i] * (float)sv[i]);
+        }
+        *reinterpret_cast<half8_t*>(op) = o;
+      }
+    }
+  }
+}
+
+}  // namespace triteia_hip

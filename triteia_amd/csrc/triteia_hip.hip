@@ -1,0 +1,339 @@
+// extern "C" boundary of libtriteia_hip.so: argument checks, launch geometry,
+// stream / device handling.  Kernels live in the headers next to this file.
+#include "../../include/triteia_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "lora.hip.h"
+#include "route_plan.hip.h"
+#include "sparse24_gemm.hip.h"
+
+namespace {
+
+using namespace triteia_hip;
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// Makes `dev` current for the duration of a call and restores the previous device.
+struct DeviceGuard {
+  int prev = -1;
+  bool ok = true;
+  explicit DeviceGuard(int dev) {
+    if (hipGetDevice(&prev) != hipSuccess) { ok = false; return; }
+    if (dev >= 0 && dev != prev) ok = hipSetDevice(dev) == hipSuccess; else prev = -1;
+  }
+  ~DeviceGuard() { if (prev >= 0) (void)hipSetDevice(prev); }
+};
+
+int check_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(TRITEIA_HIP_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+  return TRITEIA_HIP_OK;
+}
+
+int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v && *v ? atoi(v) : dflt;
+}
+
+int check_gemm_shape(int prob_m, int prob_n, int prob_k, int groupsize) {
+  if (groupsize != -1)
+    return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "groupsize=%d: only per-channel scales (groupsize=-1) are implemented", groupsize);
+  if (prob_m < 0 || prob_n < 0 || prob_k < 0 || prob_m % 128 != 0 || prob_k % 64 != 0)
+    return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "problem (m=%d, n=%d, k=%d) needs m %% 128 == 0 and k %% 64 == 0", prob_m, prob_n, prob_k);
+  return TRITEIA_HIP_OK;
+}
+
+// tokens-per-group tile of the kernel: 16 * NT rows share one pass over the weights
+int pick_nt(long tokens_per_group_hint) {
+  const int forced = env_int("TRITEIA_HIP_NT", 0);
+  if (forced == 1 || forced == 2 || forced == 4) return forced;
+  if (tokens_per_group_hint <= 16) return 1;
+  if (tokens_per_group_hint <= 32) return 2;
+  return 4;
+}
+
+template <int NT>
+void launch_nt(const Sparse24Args& a, dim3 grid, hipStream_t st) {
+  hipLaunchKernelGGL((sparse24_grouped_kernel<NT, 4>), grid, dim3(256), 0, st, a);
+}
+
+int launch_sparse24(Sparse24Args a, long tokens_per_group_hint, long max_group_tokens, hipStream_t st) {
+  if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
+  const int nt = pick_nt(tokens_per_group_hint);
+  long tsplit = (max_group_tokens + 16 * nt - 1) / (16 * nt);
+  if (tsplit < 1) tsplit = 1;
+  if (tsplit > 8) tsplit = 8;
+  const long units = (long)a.n_groups * (a.m / 128);
+  if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
+  const dim3 grid((unsigned)units, (unsigned)tsplit);
+  switch (nt) {
+    case 1: launch_nt<1>(a, grid, st); break;
+    case 2: launch_nt<2>(a, grid, st); break;
+    default: launch_nt<4>(a, grid, st); break;
+  }
+  return check_launch("sparse24_grouped_kernel");
+}
+
+void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
+                  int prob_k, int n_deltas) {
+  a.x = static_cast<const _Float16*>(A);
+  a.x_stride = prob_k;
+  a.qweight = static_cast<const uint4_t*>(B);
+  a.qweight_stride = (long)(prob_k / 32) * (prob_m / 2);
+  a.meta = static_cast<const uint4_t*>(meta);
+  a.meta_stride = (long)(prob_k / 32) * (prob_m / 4);
+  a.scales = static_cast<const _Float16*>(s);
+  a.scales_stride = prob_m;
+  a.out = static_cast<_Float16*>(C);
+  a.out_stride = prob_m;
+  a.m = prob_m;
+  a.k = prob_k;
+  a.n_deltas = n_deltas;
+  a.g_delta = a.g_start = a.g_count = a.perm = a.n_groups_dev = nullptr;
+  a.n_groups = 0;
+  a.uniform_count = 0;
+  a.delta_step = 0;
+  a.accumulate = 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int triteia_hip_version(void) { return 1000; }
+
+const char* triteia_hip_last_error(void) { return g_err; }
+
+int triteia_hip_mul_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m, int prob_n,
+                        int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k, int thread_m,
+                        int sms, int max_par) {
+  (void)workspace; (void)thread_k; (void)thread_m; (void)sms; (void)max_par;
+  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, groupsize)) return e;
+  if (prob_m == 0 || prob_n == 0 || prob_k == 0) return TRITEIA_HIP_OK;
+  if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "mul_2_4: null tensor pointer");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  Sparse24Args a;
+  fill_weights(a, A, B, meta, C, s, prob_m, prob_k, 1);
+  a.n_groups = 1;
+  a.uniform_count = prob_n;
+  return launch_sparse24(a, prob_n, prob_n, static_cast<hipStream_t>(stream));
+}
+
+int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
+                               int batch, int tokens, int prob_k, int dev, void* stream) {
+  if (int e = check_gemm_shape(prob_m, batch, prob_k, -1)) return e;
+  if (tokens < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "bmm_2_4: tokens=%d", tokens);
+  if (prob_m == 0 || batch == 0 || prob_k == 0 || tokens == 0) return TRITEIA_HIP_OK;
+  if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "bmm_2_4: null tensor pointer");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  Sparse24Args a;
+  fill_weights(a, A, B, meta, C, s, prob_m, prob_k, batch);
+  a.n_groups = batch;
+  a.uniform_count = tokens;
+  a.delta_step = 1;
+  return launch_sparse24(a, tokens, tokens, static_cast<hipStream_t>(stream));
+}
+
+int triteia_hip_bmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m, int prob_n,
+                        int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k, int thread_m,
+                        int sms, int max_par) {
+  (void)workspace; (void)thread_k; (void)thread_m; (void)sms; (void)max_par;
+  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, groupsize)) return e;
+  return triteia_hip_bmm_2_4_tokens(A, B, meta, C, s, prob_m, prob_n, 1, prob_k, dev, stream);
+}
+
+int triteia_hip_sbmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, const void* indices,
+                         const void* starts, const void* counts, int prob_m, int prob_n, int prob_k, int prob_r,
+                         int n_deltas, void* workspace, int groupsize, int dev, void* stream, int thread_k,
+                         int thread_m, int sms, int max_par) {
+  (void)workspace; (void)thread_k; (void)thread_m; (void)sms; (void)max_par;
+  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, groupsize)) return e;
+  if (prob_r < 0 || n_deltas < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sbmm_2_4: runs=%d deltas=%d", prob_r, n_deltas);
+  if (prob_m == 0 || prob_n == 0 || prob_k == 0 || prob_r == 0) return TRITEIA_HIP_OK;
+  if (!A || !B || !meta || !C || !s || !indices || !starts || !counts)
+    return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4: null tensor pointer");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  Sparse24Args a;
+  fill_weights(a, A, B, meta, C, s, prob_m, prob_k, n_deltas);
+  a.g_delta = static_cast<const int*>(indices);
+  a.g_start = static_cast<const int*>(starts);
+  a.g_count = static_cast<const int*>(counts);
+  a.n_groups = prob_r;
+  const long hint = (4L * prob_n + prob_r - 1) / prob_r;
+  return launch_sparse24(a, hint, prob_n, static_cast<hipStream_t>(stream));
+}
+
+size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n_deltas) {
+  if (prob_n < 0 || n_deltas < 0) return 0;
+  return sizeof(int) * (size_t)plan_layout(prob_n, n_deltas).total;
+}
+
+int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
+                           size_t workspace_bytes, int dev, void* stream) {
+  if (prob_n < 0 || n_deltas < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "route_plan: tokens=%d deltas=%d", prob_n, n_deltas);
+  if (n_deltas > kPlanMaxDeltas)
+    return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "route_plan: at most %d deltas per call (got %d)", kPlanMaxDeltas, n_deltas);
+  if (!workspace || workspace_bytes < triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas))
+    return fail(TRITEIA_HIP_ERR_ARGUMENT, "route_plan: workspace must hold %zu bytes (got %zu)",
+                triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas), workspace_bytes);
+  if (prob_n > 0 && !token_indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "route_plan: null indices");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  hipLaunchKernelGGL(route_plan_kernel, dim3(1), dim3(kPlanThreads), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const int*>(token_indices), prob_n, n_deltas, index_offset, static_cast<int*>(workspace));
+  return check_launch("route_plan_kernel");
+}
+
+int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                const void* token_indices, int index_offset, int n_deltas, int prob_m, int prob_n,
+                                int prob_k, void* workspace, size_t workspace_bytes, int accumulate, int dev,
+                                void* stream) {
+  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, -1)) return e;
+  if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: accumulate=%d", accumulate);
+  if (prob_m == 0 || prob_n == 0 || prob_k == 0 || n_deltas == 0) return TRITEIA_HIP_OK;
+  if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null tensor pointer");
+  if (int e = triteia_hip_route_plan(token_indices, index_offset, n_deltas, prob_n, workspace, workspace_bytes, dev, stream))
+    return e;
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  const PlanLayout L = plan_layout(prob_n, n_deltas);
+  const int* ws = static_cast<const int*>(workspace);
+  Sparse24Args a;
+  fill_weights(a, A, B, meta, C, s, prob_m, prob_k, n_deltas);
+  a.g_delta = ws + L.g_delta;
+  a.g_start = ws + L.g_start;
+  a.g_count = ws + L.g_count;
+  a.perm = ws + L.perm;
+  a.n_groups_dev = ws + L.header;
+  a.n_groups = prob_n < n_deltas ? prob_n : n_deltas;
+  a.accumulate = accumulate;
+  const long hint = (4L * prob_n + a.n_groups - 1) / a.n_groups;
+  return launch_sparse24(a, hint, prob_n, static_cast<hipStream_t>(stream));
+}
+
+int triteia_hip_bgmv(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                     int num_layers, int layer_idx, float scale, int dev, void* stream) {
+  if (batch < 0 || h_in <= 0 || h_out <= 0 || num_layers <= 0 || layer_idx < 0 || layer_idx >= num_layers)
+    return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "bgmv: batch=%d h_in=%d h_out=%d layers=%d layer=%d", batch, h_in, h_out, num_layers, layer_idx);
+  const int narrow = h_in < h_out ? h_in : h_out;
+  if (h_in % 8 != 0 || h_out % 8 != 0 || narrow > kLoraMaxNarrow)
+    return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "No suitable kernel. h_in=%d h_out=%d", h_in, h_out);
+  if (batch == 0) return TRITEIA_HIP_OK;
+  if (!Y || !X || !W || !indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "bgmv: null tensor pointer");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (h_in >= h_out) {
+    hipLaunchKernelGGL(bgmv_shrink_kernel, dim3(batch), dim3(256), 0, st, static_cast<_Float16*>(Y),
+                       static_cast<const _Float16*>(X), static_cast<const _Float16*>(W),
+                       static_cast<const long long*>(indices), h_in, h_out, (long)num_layers, (long)layer_idx, scale);
+  } else {
+    hipLaunchKernelGGL(bgmv_expand_kernel, dim3((h_out + 255) / 256, batch), dim3(256), 0, st, static_cast<_Float16*>(Y),
+                       static_cast<const _Float16*>(X), static_cast<const _Float16*>(W),
+                       static_cast<const long long*>(indices), h_in, h_out, (long)num_layers, (long)layer_idx, scale);
+  }
+  return check_launch("bgmv kernel");
+}
+
+size_t triteia_hip_sgmv_tmp_size(int num_problems) {
+  // the reference's CUTLASS argument block: 60 bytes per problem (sgmv.cuh:48-52)
+  return num_problems > 0 ? (size_t)60 * (size_t)num_problems : 0;
+}
+
+static int launch_sgmv(SgmvArgs a, int max_rows, hipStream_t st) {
+  const int narrow = a.d_in < a.d_out ? a.d_in : a.d_out;
+  if (a.d_in % 8 != 0 || a.d_out % 8 != 0 || narrow > kLoraMaxNarrow)
+    return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "No suitable kernel. d_in=%d d_out=%d", a.d_in, a.d_out);
+  if (a.n_groups <= 0) return TRITEIA_HIP_OK;
+  if (a.d_in >= a.d_out) {
+    int row_tiles = (max_rows + 3) / 4;
+    if (row_tiles > 64) row_tiles = 64;
+    if (row_tiles < 1) row_tiles = 1;
+    hipLaunchKernelGGL((sgmv_shrink_kernel<4>), dim3(a.n_groups, row_tiles), dim3(256), 0, st, a);
+  } else {
+    const dim3 grid(a.n_groups, (a.d_out + 255) / 256);
+    if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_kernel<16>), grid, dim3(256), 0, st, a);
+    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_kernel<32>), grid, dim3(256), 0, st, a);
+    else if (a.d_in <= 64) hipLaunchKernelGGL((sgmv_expand_kernel<64>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((sgmv_expand_kernel<128>), grid, dim3(256), 0, st, a);
+  }
+  return check_launch("sgmv kernel");
+}
+
+int triteia_hip_sgmv(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
+                     int d_out, int layer_idx, int dev, void* stream) {
+  (void)tmp;
+  if (num_problems < 0 || d_in <= 0 || d_out <= 0 || layer_idx < 0)
+    return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sgmv: problems=%d d_in=%d d_out=%d layer=%d", num_problems, d_in, d_out, layer_idx);
+  if (num_problems == 0) return TRITEIA_HIP_OK;
+  if (!y || !x || !w_ptrs || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sgmv: null tensor pointer");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  SgmvArgs a;
+  memset(&a, 0, sizeof(a));
+  a.y = static_cast<_Float16*>(y);
+  a.y_stride = d_out;
+  a.x = static_cast<const _Float16*>(x);
+  a.x_stride = d_in;
+  a.d_in = d_in;
+  a.d_out = d_out;
+  a.w_ptrs = static_cast<const long long*>(w_ptrs);
+  a.layer_off = (long)layer_idx * d_in * d_out;
+  a.seg = static_cast<const int*>(s);
+  a.n_groups = num_problems;
+  a.n_adapters = num_problems;
+  a.scale = 1.0f;
+  // segment lengths live on the device; size the row-tile dimension for a few rows per segment
+  return launch_sgmv(a, 16, static_cast<hipStream_t>(stream));
+}
+
+int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
+                            int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
+                            int dev, void* stream) {
+  if (prob_n < 0 || n_adapters < 0 || d_in <= 0 || d_out <= 0)
+    return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sgmv_routed: tokens=%d adapters=%d d_in=%d d_out=%d", prob_n, n_adapters, d_in, d_out);
+  if (prob_n == 0 || n_adapters == 0) return TRITEIA_HIP_OK;
+  if (!y || !x || !w_base || !plan) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sgmv_routed: null tensor pointer");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  const PlanLayout L = plan_layout(prob_n, n_adapters);
+  const int* ws = static_cast<const int*>(plan);
+  SgmvArgs a;
+  memset(&a, 0, sizeof(a));
+  a.y = static_cast<_Float16*>(y);
+  a.y_stride = y_stride;
+  a.x = static_cast<const _Float16*>(x);
+  a.x_stride = x_stride;
+  a.d_in = d_in;
+  a.d_out = d_out;
+  a.w_base = static_cast<const _Float16*>(w_base);
+  a.w_stride = w_stride;
+  a.g_delta = ws + L.g_delta;
+  a.g_start = ws + L.g_start;
+  a.g_count = ws + L.g_count;
+  a.perm = ws + L.perm;
+  a.n_groups_dev = ws + L.header;
+  a.n_groups = prob_n < n_adapters ? prob_n : n_adapters;
+  a.n_adapters = n_adapters;
+  a.scale = scale;
+  return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,93 @@
+"""ctypes binding of libtriteia_hip.so (declared in include/triteia_hip.h).
+
+The library is built in-tree by `python -m triteia_amd.build`; there is no
+fallback implementation: if it cannot be loaded every op raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "..", "lib", "libtriteia_hip.so"))
+
+ERR_PROB_SHAPE = 1
+ERR_KERN_SHAPE = 2
+ERR_ARGUMENT = 3
+ERR_RUNTIME = 4
+
+_c_int, _c_vp, _c_sz, _c_long, _c_float = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_long, ctypes.c_float
+
+# name -> (restype, argtypes); mirrors include/triteia_hip.h one to one
+SIGNATURES = {
+    "triteia_hip_version": (_c_int, []),
+    "triteia_hip_last_error": (ctypes.c_char_p, []),
+    "triteia_hip_mul_2_4": (_c_int, [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
+    "triteia_hip_bmm_2_4": (_c_int, [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
+    "triteia_hip_bmm_2_4_tokens": (_c_int, [_c_vp] * 5 + [_c_int] * 4 + [_c_int, _c_vp]),
+    "triteia_hip_sbmm_2_4": (_c_int, [_c_vp] * 8 + [_c_int] * 5 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
+    "triteia_hip_sbmm_2_4_routed": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_vp, _c_sz, _c_int, _c_int, _c_vp]),
+    "triteia_hip_sbmm_routed_workspace_bytes": (_c_sz, [_c_int, _c_int]),
+    "triteia_hip_route_plan": (_c_int, [_c_vp, _c_int, _c_int, _c_int, _c_vp, _c_sz, _c_int, _c_vp]),
+    "triteia_hip_bgmv": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_float, _c_int, _c_vp]),
+    "triteia_hip_sgmv": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp]),
+    "triteia_hip_sgmv_tmp_size": (_c_sz, [_c_int]),
+    "triteia_hip_sgmv_routed": (_c_int, [_c_vp, _c_long, _c_vp, _c_long, _c_vp, _c_long] + [_c_int] * 3
+                                + [_c_float, _c_vp, _c_int, _c_int, _c_vp]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises RuntimeError if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} not found: build it with `python -m triteia_amd.build` "
+                "(there is no fallback implementation)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    return lib().triteia_hip_last_error().decode("utf-8", "replace")
+
+
+def stream_of(t: torch.Tensor):
+    """Handle of torch's current stream on the tensor's device."""
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def device_index(t: torch.Tensor) -> int:
+    return t.device.index if t.device.index is not None else torch.cuda.current_device()
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def require_gpu(**tensors):
+    dev = None
+    for name, t in tensors.items():
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{name} must be a torch.Tensor")
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be a GPU tensor (this op has no CPU implementation)")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"{name} is on {t.device}, expected {dev}")
+
+
+def require_dtype(t, dtype, name):
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
