@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Benchmark of the multi-model low-precision GEMM path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg0..cfg4] [--tokens T]
+
+A step is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM: for the default workload (indexed sbmm, 64 tokens routed over 16 deltas of
+4096x4096) one call of `triteia_hip_sbmm_2_4_routed` (routing kernel + grouped sparse-MFMA
+kernel).  Successive steps rotate over enough distinct copies of the packed deltas that the
+weights come from HBM, not from the 256 MB Infinity Cache.
+
+Prints ONE JSON line.  `value` is dense-equivalent TFLOP/s (2 * routed_tokens * k * m per
+step, the reference's convention, meta/benchmarks/bench_sbmm.py:17) over the timed region;
+`roofline` scores the dominant kernel against HBM bandwidth with its duration measured live by
+HIP events; `cpu_baseline` is the CPU oracle (dequantise, then torch matmul per delta) timed on
+the host cores on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_SPARSE_F16_TFLOPS = 5000.0  # 2:4 sparse fp16 (dense fp16 2.5 PFLOP/s), dense-equivalent FLOPs
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
+    p.add_argument("--tokens", type=int, default=None, help="override the token count (cfg2/cfg3/cfg4)")
+    p.add_argument("--deltas", type=int, default=None, help="override the number of resident deltas (cfg4)")
+    p.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = auto)")
+    p.add_argument("--no-graph", action="store_true", help="time eager launches instead of one captured HIP graph")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--warm-cache", action="store_true", help="do not rotate weight copies (Infinity-Cache-warm number)")
+    return p.parse_args()
+
+
+class Problem:
+    """Device tensors + bound C-ABI calls for one workload."""
+
+    def __init__(self, wl, copies, torch, ffi):
+        from triteia_amd import workloads as W
+        self.wl, self.torch, self.ffi = wl, torch, ffi
+        dev = "cuda:0"
+        self.dev = dev
+        self.lib = ffi.lib()
+        self.copies = copies
+        self.weights = [W.random_packed_deltas(wl.n_deltas, wl.k, wl.m, wl.seed + 7919 * c, dev) for c in range(copies)]
+        self.x = W.random_activations(wl.tokens, wl.k, wl.seed + 1, dev)
+        self.out = torch.zeros((wl.tokens, wl.m), dtype=torch.float16, device=dev)
+        self.idx = torch.from_numpy(wl.indices).to(dev) if wl.indices is not None else None
+        nbytes = self.lib.triteia_hip_sbmm_routed_workspace_bytes(wl.tokens, wl.n_deltas)
+        self.ws = torch.zeros((nbytes + 3) // 4, dtype=torch.int32, device=dev)
+        self.ws_bytes = self.ws.numel() * 4
+        self.lock_ws = torch.zeros(max(wl.m, 16) * max(1, wl.n_deltas), dtype=torch.int32, device=dev)
+        if wl.op == "ldmm":
+            g = torch.Generator(device=dev).manual_seed(wl.seed + 3)
+            self.base = [(torch.randn((wl.m, wl.k), generator=g, device=dev) * 0.02).half() for _ in range(copies)]
+            self.lora_a = (torch.randn((wl.n_lora, wl.k, wl.lora_rank), generator=g, device=dev) * 0.01).half()
+            self.lora_b = (torch.randn((wl.n_lora, wl.lora_rank, wl.m), generator=g, device=dev) * 0.01).half()
+            self.v = torch.zeros((wl.tokens, wl.lora_rank), dtype=torch.float16, device=dev)
+
+    def _chk(self, rc):
+        if rc != 0:
+            raise RuntimeError(f"triteia_hip call failed ({rc}): {self.ffi.last_error()}")
+
+    def stream(self):
+        return ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+
+    def plan(self):
+        wl, P = self.wl, self.ffi.ptr
+        self._chk(self.lib.triteia_hip_route_plan(P(self.idx), 0, wl.n_deltas, wl.tokens, P(self.ws), self.ws_bytes, 0, self.stream()))
+
+    def delta_kernel(self, i, accumulate=0):
+        """Only the dominant kernel (on an existing plan for sbmm / ldmm)."""
+        wl, P = self.wl, self.ffi.ptr
+        q, me, s = self.weights[i % self.copies]
+        st = self.stream()
+        if wl.op == "matmul":
+            self._chk(self.lib.triteia_hip_mul_2_4(P(self.x), P(q), P(me), P(self.out), P(s), wl.m, wl.tokens, wl.k, P(self.lock_ws),
+                                                    -1, 0, st, -1, -1, -1, 16))
+        elif wl.op == "bmm":
+            self._chk(self.lib.triteia_hip_bmm_2_4(P(self.x), P(q), P(me), P(self.out), P(s), wl.m, wl.n_deltas, wl.k, P(self.lock_ws),
+                                                    -1, 0, st, -1, -1, -1, 16))
+        else:
+            self._chk(self.lib.triteia_hip_sbmm_2_4_planned(P(self.x), P(q), P(me), P(self.out), P(s), P(self.ws), wl.n_deltas, wl.m,
+                                                            wl.tokens, wl.k, accumulate, 0, st))
+
+    def step(self, i):
+        """The whole hot path for one batch."""
+        wl, P, torch = self.wl, self.ffi.ptr, self.torch
+        if wl.op in ("matmul", "bmm"):
+            self.delta_kernel(i)
+        elif wl.op == "sbmm":
+            q, me, s = self.weights[i % self.copies]
+            self._chk(self.lib.triteia_hip_sbmm_2_4_routed(P(self.x), P(q), P(me), P(self.out), P(s), P(self.idx), 0, wl.n_deltas, wl.m,
+                                                           wl.tokens, wl.k, P(self.ws), self.ws_bytes, 0, 0, self.stream()))
+        else:  # ldmm: dense base GEMM (library) + routed LoRA (SGMV) + routed delta, one routing plan for both
+            torch.matmul(self.x, self.base[i % self.copies].t(), out=self.out)
+            self.plan()
+            self.v.zero_()
+            st = self.stream()
+            r = wl.lora_rank
+            self._chk(self.lib.triteia_hip_sgmv_routed(P(self.v), r, P(self.x), wl.k, P(self.lora_a), wl.k * r, wl.n_lora, wl.k, r,
+                                                       1.0, P(self.ws), wl.tokens, 0, st))
+            self._chk(self.lib.triteia_hip_sgmv_routed(P(self.out), wl.m, P(self.v), r, P(self.lora_b), r * wl.m, wl.n_lora, r, wl.m,
+                                                       1.0, P(self.ws), wl.tokens, 0, st))
+            self.delta_kernel(i, accumulate=1)
+
+
+def cpu_baseline(wl, torch, budget_s=20.0):
+    """The CPU oracle on the host cores: numpy dequantise of packed deltas + torch matmul per
+    delta, on as many of the workload's deltas as fit the time budget, scaled to all of them."""
+    from oracle import triteia_oracle as orc
+    from triteia_amd import workloads as W
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    used = sorted(set(int(i) for i in wl.indices if i >= 0)) if wl.indices is not None else list(range(wl.n_deltas))
+    counts = {d: (int((wl.indices == d).sum()) if wl.indices is not None else wl.tokens // wl.n_deltas) for d in used}
+    x = W.random_activations(wl.tokens, wl.k, wl.seed + 1, "cpu").float()
+    t_deq = t_mm = 0.0
+    flops = 0.0
+    done = 0
+    t_begin = time.perf_counter()
+    for d in used:
+        q, me, s = W.random_packed_deltas(1, wl.k, wl.m, wl.seed + 31 * d, "cpu")
+        t0 = time.perf_counter()
+        dense = orc.unpack(q[0].numpy(), me[0].numpy(), s[0].numpy())
+        t1 = time.perf_counter()
+        wt = torch.from_numpy(dense).float()
+        rows = x[: counts[d]]
+        y = rows @ wt
+        t2 = time.perf_counter()
+        del y
+        t_deq += t1 - t0
+        t_mm += t2 - t1
+        flops += 2.0 * counts[d] * wl.k * wl.m
+        done += 1
+        if time.perf_counter() - t_begin > budget_s:
+            break
+    total = t_deq + t_mm
+    return {
+        "value": round(flops / total / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"{done} of {len(used)} routed deltas of the workload (numpy dequantise {t_deq:.2f}s on 1 thread + torch fp32 "
+                  f"matmul {t_mm:.3f}s on {cores} threads); the rate is per delta and carries over to all of them",
+        "dequant_s": round(t_deq, 3), "matmul_s": round(t_mm, 4),
+    }
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives in this path); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from triteia_amd import workloads as W
+    from triteia_amd.python.capi import _ffi as ffi
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    ffi.lib()   # fails loudly if the HIP library is missing
+
+    wl = W.config(a.workload, a.tokens)
+    if a.deltas is not None and a.workload == "cfg4":
+        wl.n_deltas = a.deltas
+        wl.indices = W.zipf_indices(wl.tokens, wl.n_deltas, 1.2, wl.seed)
+    touched = wl.distinct_deltas() * wl.delta_bytes
+    if a.warm_cache:
+        copies = 1
+    elif a.copies > 0:
+        copies = a.copies
+    else:
+        # enough distinct bytes to out-run the 256 MB Infinity Cache, within ~12 GB
+        copies = max(1, min(64, int(np.ceil(1.5 * 2 ** 30 / max(touched, 1))), int(12 * 2 ** 30 // (wl.n_deltas * wl.delta_bytes)) or 1))
+    prob = Problem(wl, copies, torch, ffi)
+    torch.cuda.synchronize()
+
+    # ---- whole-job timing: W warm-up steps, then exactly K steps
+    for i in range(a.warmup):
+        prob.step(i)
+    torch.cuda.synchronize()
+    use_graph = not a.no_graph
+    if use_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(a.steps):
+                    prob.step(a.warmup + i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    else:
+        t0 = time.perf_counter()
+        for i in range(a.steps):
+            prob.step(a.warmup + i)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    # eager launches too (shows the host launch cost next to the graph number)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        prob.step(a.warmup + i)
+    torch.cuda.synchronize()
+    eager = time.perf_counter() - t0
+
+    ms_per_step = elapsed / a.steps * 1e3
+    flops = wl.delta_flops()
+    if wl.op == "ldmm":
+        flops += 2.0 * wl.tokens * wl.k * wl.m + 2.0 * wl.routed_tokens() * wl.lora_rank * (wl.k + wl.m)
+    value = flops / (elapsed / a.steps) / 1e12
+
+    # ---- dominant kernel alone: HIP events on the launch stream, batches of back-to-back launches
+    if wl.indices is not None:
+        prob.plan()
+    for i in range(5):
+        prob.delta_kernel(i)
+    torch.cuda.synchronize()
+    batch, reps = 10, max(3, min(20, a.steps // 10))
+    durs = []
+    for r in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(batch):
+            prob.delta_kernel(r * batch + i)
+        e1.record()
+        e1.synchronize()
+        durs.append(e0.elapsed_time(e1) / batch * 1e-3)
+    kdur = float(np.median(durs))
+    abytes = wl.delta_algorithmic_bytes()
+    achieved = abytes / kdur / 1e9
+    kflops = wl.delta_flops() / kdur / 1e12
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", f"traffic_{a.workload}.json")
+    if os.path.exists(tpath) and a.tokens is None and a.deltas is None:
+        try:
+            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        except Exception:
+            traffic = None
+    roofline = {
+        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": traffic, "kernel": "sparse24_grouped_kernel", "kernel_us": round(kdur * 1e6, 2), "algorithmic_bytes": abytes,
+        "kernel_tflops": round(kflops, 2), "mfma_frac": round(kflops / MFMA_SPARSE_F16_TFLOPS, 4),
+    }
+
+    res = {
+        "metric": "sbmm/ldmm dense-equivalent TFLOP/s at Llama-2-7B shapes (with % of HBM roofline)",
+        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (int4 2:4 weights, fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": wl.name, "op": wl.op, "k": wl.k, "m": wl.m, "deltas_resident": wl.n_deltas, "deltas_used": wl.distinct_deltas(),
+                   "tokens": wl.tokens, "tokens_routed": wl.routed_tokens(), "weight_copies_rotated": copies,
+                   "launch": "hip-graph" if use_graph else "eager"},
+        "eager_ms_per_step": round(eager / a.steps * 1e3, 5),
+        "step_gbs": round((abytes + (wl.k * wl.m * 2 if wl.op == "ldmm" else 0)) / (elapsed / a.steps) / 1e9, 1),
+        "roofline": roofline,
+    }
+    if not a.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(wl, torch)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

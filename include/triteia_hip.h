@@ -112,6 +112,14 @@ TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n
 TRITEIA_HIP_API int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
                            size_t workspace_bytes, int dev, void* stream);
 
+/* The multiply step alone, on a plan made by triteia_hip_route_plan for the same
+ * (prob_n, n_deltas): C[t] (+)= A[t] @ dequant(B[d]) for every routed token.  One
+ * plan serves every layer of a forward pass (the routing of a batch does not
+ * change between layers) and the LoRA path.  No counterpart in the reference. */
+TRITEIA_HIP_API int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                 const void* plan, int n_deltas, int prob_m, int prob_n, int prob_k, int accumulate,
+                                 int dev, void* stream);
+
 /* BGMV: Y[b, :] += scale * W[indices[b] * num_layers + layer_idx] @ X[b, :]
  * with W [n, num_layers, h_out, h_in] fp16 (out-major) and indices int64 [batch]
  * (negative = skip).  Replaces bgmv_kernel<feat_in, feat_out, T>

@@ -201,20 +201,18 @@ int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_de
   return check_launch("route_plan_kernel");
 }
 
-int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, void* C, const void* s,
-                                const void* token_indices, int index_offset, int n_deltas, int prob_m, int prob_n,
-                                int prob_k, void* workspace, size_t workspace_bytes, int accumulate, int dev,
-                                void* stream) {
+int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                 const void* plan, int n_deltas, int prob_m, int prob_n, int prob_k, int accumulate,
+                                 int dev, void* stream) {
   if (int e = check_gemm_shape(prob_m, prob_n, prob_k, -1)) return e;
-  if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: accumulate=%d", accumulate);
+  if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_planned: accumulate=%d", accumulate);
+  if (n_deltas < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sbmm_2_4_planned: deltas=%d", n_deltas);
   if (prob_m == 0 || prob_n == 0 || prob_k == 0 || n_deltas == 0) return TRITEIA_HIP_OK;
-  if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null tensor pointer");
-  if (int e = triteia_hip_route_plan(token_indices, index_offset, n_deltas, prob_n, workspace, workspace_bytes, dev, stream))
-    return e;
+  if (!A || !B || !meta || !C || !s || !plan) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_planned: null tensor pointer");
   DeviceGuard g(dev);
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   const PlanLayout L = plan_layout(prob_n, n_deltas);
-  const int* ws = static_cast<const int*>(workspace);
+  const int* ws = static_cast<const int*>(plan);
   Sparse24Args a;
   fill_weights(a, A, B, meta, C, s, prob_m, prob_k, n_deltas);
   a.g_delta = ws + L.g_delta;
@@ -226,6 +224,19 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   a.accumulate = accumulate;
   const long hint = (4L * prob_n + a.n_groups - 1) / a.n_groups;
   return launch_sparse24(a, hint, prob_n, static_cast<hipStream_t>(stream));
+}
+
+int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                const void* token_indices, int index_offset, int n_deltas, int prob_m, int prob_n,
+                                int prob_k, void* workspace, size_t workspace_bytes, int accumulate, int dev,
+                                void* stream) {
+  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, -1)) return e;
+  if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: accumulate=%d", accumulate);
+  if (prob_m == 0 || prob_n == 0 || prob_k == 0 || n_deltas == 0) return TRITEIA_HIP_OK;
+  if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null tensor pointer");
+  if (int e = triteia_hip_route_plan(token_indices, index_offset, n_deltas, prob_n, workspace, workspace_bytes, dev, stream))
+    return e;
+  return triteia_hip_sbmm_2_4_planned(A, B, meta, C, s, workspace, n_deltas, prob_m, prob_n, prob_k, accumulate, dev, stream);
 }
 
 int triteia_hip_bgmv(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,

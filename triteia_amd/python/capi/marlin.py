@@ -169,3 +169,25 @@ def sbmm_2_4_routed(A, B, meta, C, s, token_indices, index_offset=0, accumulate=
         workspace.numel() * workspace.element_size(), 1 if accumulate else 0, _ffi.device_index(A), _ffi.stream_of(A))
     _raise(err, prob_m, prob_n, prob_k, -1, -1, -1)
     return workspace
+
+
+def sbmm_2_4_planned(A, B, meta, C, s, plan, accumulate=False):
+    """The multiply step of `sbmm_2_4_routed` on an existing routing plan (from `route_plan`
+    with n_deltas = B.shape[0] and as many tokens as A has rows); lets one plan serve many
+    layers."""
+    _gemm_checks(A, B, meta, C, s)
+    _ffi.require_gpu(plan=plan)
+    if A.dim() != 2 or C.dim() != 2 or B.dim() != 3:
+        raise RuntimeError("A and C must be 2-D, B 3-D")
+    prob_n, prob_k = A.shape
+    prob_m = C.shape[1]
+    n_deltas = B.shape[0]
+    need = _ffi.lib().triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas)
+    if plan.numel() * plan.element_size() < need:
+        raise RuntimeError(f"plan holds {plan.numel() * plan.element_size()} bytes, {need} needed")
+    if prob_m % 128 == 0 and prob_k % 64 == 0:
+        _check_packed(B, meta, s, prob_m, prob_k, lead=(n_deltas,))
+    err = _ffi.lib().triteia_hip_sbmm_2_4_planned(
+        _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), _ffi.ptr(plan), n_deltas, prob_m, prob_n,
+        prob_k, 1 if accumulate else 0, _ffi.device_index(A), _ffi.stream_of(A))
+    _raise(err, prob_m, prob_n, prob_k, -1, -1, -1)
