@@ -74,6 +74,10 @@ struct Sparse24Args {
   int delta_step;
   int n_deltas;             // deltas with index outside [0, n_deltas) are skipped
   int accumulate;           // 0: out = result, 1: out += result
+  int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run
+#ifdef TRITEIA_HIP_TIMELINE
+  long long* timeline;      // [unit][wave][4] 100 MHz timestamps (debug builds only)
+#endif
 };
 
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
@@ -91,6 +95,14 @@ __device__ __forceinline__ uint32_t dequant_odd(uint32_t w) {
   return h2_bits(bits_h2((w & 0x00f000f0u) | 0x64006400u) * mul + add);
 }
 
+// Workgroup barrier that orders LDS traffic only: outstanding global loads (the prefetch
+// ring) are not waited for.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 template <int NT>
 struct StepFrag {
   uint4_t wq[4];        // weights: groups a and a+4 (a = vector index) of 8 columns
@@ -101,18 +113,23 @@ struct StepFrag {
 
 constexpr int kRedStride = 132;  // floats per token row in the reduction buffer (128 + pad)
 
-template <int NT, int KW>
+template <int NT, int KW, int DEPTH>
 __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse24Args p) {
   __shared__ float red[KW][16][kRedStride];
   __shared__ int s_rows[16 * NT];
 
+#ifdef TRITEIA_HIP_TIMELINE
+  const long long ts_entry = wall_clock64();
+#endif
   const int col_blocks = p.m >> 7;
   const int unit = blockIdx.x;
   const int grp = unit / col_blocks;
-  const int cb = unit - grp * col_blocks;
-  const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
-  if (grp >= n_groups) return;
-
+  int cb = unit - grp * col_blocks;
+  // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): give every XCD a
+  // contiguous run of column blocks instead of every 8th one.
+  if (p.xcd_swizzle && (col_blocks & 7) == 0) cb = (cb & 7) * (col_blocks >> 3) + (cb >> 3);
+  // group descriptor and live group count are fetched side by side (no dependent chain);
+  // grp < p.n_groups (the host's upper bound) keeps the descriptor reads in bounds
   int delta, start, count;
   if (p.g_delta) {
     delta = p.g_delta[grp];
@@ -123,6 +140,8 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
     start = grp * p.uniform_count;
     count = p.uniform_count;
   }
+  const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
+  if (grp >= n_groups) return;
   if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
 
   const int tid = threadIdx.x;
@@ -140,24 +159,48 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
   const uint4_t* mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (r >> 3)) * 16 + (r & 7);
   const _Float16* sc = p.scales + (long)delta * p.scales_stride + cb * 128;
 
+  // Steps past the end of K (st >= n_steps) read step 0 again: cheap cache hits that keep the
+  // load count per iteration constant; they are never multiplied.
+  auto load_w = [&](StepFrag<NT>& f, int st) {
+    const int tr0 = (st < n_steps ? st : 0) << 2;
+    const int tr = min(tr0 + q, k_rows - 1);  // clamped: rows past the end are cancelled by zero B
+    const uint4_t* wp = qw_lane + (long)tr * qrow;
+    const uint4_t* mp = mt_lane + (long)tr * mrow;
+#pragma unroll
+    for (int a = 0; a < 4; a++) f.wq[a] = wp[a];
+    f.mt[0] = mp[0];
+    f.mt[1] = mp[8];
+  };
+
   // blockIdx.y splits a group's tokens between workgroups (each re-streams the weights)
   for (int t0 = blockIdx.y * 16 * NT; t0 < count; t0 += gridDim.y * 16 * NT) {
     const int cnt = min(count - t0, 16 * NT);
-    __syncthreads();  // previous pass finished reading s_rows / red
-    if (tid < 16 * NT) {
-      int row = -1;
-      if (tid < cnt) row = p.perm ? p.perm[start + t0 + tid] : start + t0 + tid;
-      s_rows[tid] = row;
+    // Start-up order matters (vector loads return in order): first the tiny per-lane read of
+    // this lane's token rows, then the weight stream (which only needs the delta id), and the
+    // activation loads once the rows have arrived.  No barrier is needed before the K loop.
+    int rows[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const int slot = min(nt * 16 + r, cnt - 1);   // slots past the end re-read the last row
+      rows[nt] = p.perm ? p.perm[start + t0 + slot] : start + t0 + slot;
     }
-    __syncthreads();
+    StepFrag<NT> ring[DEPTH];
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) load_w(ring[j], wave + j * KW);
 
+    // Every lane always loads from a valid address, so that the number of loads per step is
+    // fixed and the hardware load counter can be waited on exactly (the output columns of the
+    // duplicated slots are never stored).
     const _Float16* xrow[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
-      const int row = s_rows[nt * 16 + r];
       // B operand slot layout: this lane supplies k offsets 8*(q%2) + {0..7} of
       // packed rows tr0 + q/2 and tr0 + 2 + q/2
-      xrow[nt] = row >= 0 ? p.x + (long)row * p.x_stride + 32 * (q >> 1) + 8 * (q & 1) : nullptr;
+      xrow[nt] = p.x + (long)rows[nt] * p.x_stride + 32 * (q >> 1) + 8 * (q & 1);
+    }
+    if (wave == 0 && q == 0) {
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) s_rows[nt * 16 + r] = (nt * 16 + r < cnt) ? rows[nt] : -1;
     }
 
     float4_t acc[8][NT];
@@ -166,36 +209,25 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) acc[c][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    auto load_step = [&](StepFrag<NT>& f, int st) {
-      const int tr0 = st << 2;
-      const int tr = min(tr0 + q, k_rows - 1);  // clamped: rows past the end are cancelled by zero B
-      const uint4_t* wp = qw_lane + (long)tr * qrow;
-#pragma unroll
-      for (int a = 0; a < 4; a++) f.wq[a] = __builtin_nontemporal_load(wp + a);
-      const uint4_t* mp = mt_lane + (long)tr * mrow;
-      f.mt[0] = __builtin_nontemporal_load(mp);
-      f.mt[1] = __builtin_nontemporal_load(mp + 8);
-      const bool ok_a = (tr0 + (q >> 1)) < k_rows;
-      const bool ok_b = (tr0 + 2 + (q >> 1)) < k_rows;
+    auto load_x = [&](StepFrag<NT>& f, int st) {
+      const int tr0 = (st < n_steps ? st : 0) << 2;
+      // rows tr0+2.. may lie past the end of K in the last step: clamp the address, zero at use
+      const long xoff_a = (long)min(tr0, k_rows - 1 - (q >> 1)) * 32;
+      const long xoff_b = (long)min(tr0 + 2, k_rows - 1 - (q >> 1)) * 32;
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        const uint4_t zero = {0u, 0u, 0u, 0u};
-        f.xa[nt][0] = f.xa[nt][1] = f.xb[nt][0] = f.xb[nt][1] = zero;
-        if (xrow[nt] != nullptr && nt * 16 < cnt) {
-          const _Float16* xp = xrow[nt] + (long)tr0 * 32;
-          if (ok_a) {
-            f.xa[nt][0] = *reinterpret_cast<const uint4_t*>(xp);
-            f.xa[nt][1] = *reinterpret_cast<const uint4_t*>(xp + 16);
-          }
-          if (ok_b) {
-            f.xb[nt][0] = *reinterpret_cast<const uint4_t*>(xp + 64);
-            f.xb[nt][1] = *reinterpret_cast<const uint4_t*>(xp + 80);
-          }
-        }
+        f.xa[nt][0] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_a);
+        f.xa[nt][1] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_a + 16);
+        f.xb[nt][0] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_b);
+        f.xb[nt][1] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_b + 16);
       }
     };
 
-    auto compute_step = [&](const StepFrag<NT>& f) {
+    auto compute_step = [&](const StepFrag<NT>& f, int st) {
+      const int tr0 = st << 2;
+      const bool tail = tr0 + 4 > k_rows;            // wave-uniform: only the last, partial step
+      const bool ok_a = (tr0 + (q >> 1)) < k_rows;
+      const bool ok_b = (tr0 + 2 + (q >> 1)) < k_rows;
 #pragma unroll
       for (int u = 0; u < 2; u++) {
         half16_t b[NT];
@@ -204,6 +236,13 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
           typedef uint32_t uint8_t_v __attribute__((ext_vector_type(8)));
           uint8_t_v bb = {f.xa[nt][u][0], f.xa[nt][u][1], f.xa[nt][u][2], f.xa[nt][u][3],
                           f.xb[nt][u][0], f.xb[nt][u][1], f.xb[nt][u][2], f.xb[nt][u][3]};
+          if (tail) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+              if (!ok_a) bb[i] = 0u;
+              if (!ok_b) bb[4 + i] = 0u;
+            }
+          }
           b[nt] = __builtin_bit_cast(half16_t, bb);
         }
 #pragma unroll
@@ -232,23 +271,33 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
       }
     };
 
-    // K loop: wave w takes steps w, w + KW, ...; one step of register prefetch
-    StepFrag<NT> cur, nxt;
-    int st = wave;
-    if (st < n_steps) load_step(cur, st);
-    while (st < n_steps) {
-      const int st_next = st + KW;
-      if (st_next < n_steps) load_step(nxt, st_next);
-      compute_step(cur);
-      cur = nxt;
-      st = st_next;
+    // K loop: wave w takes steps w, w + KW, ...; DEPTH steps of loads are kept in flight in
+    // registers (ring of fragments, statically indexed through the unrolled inner loop).
+    // The body is branch-free apart from the wave-uniform "is this step real" test around the
+    // arithmetic, so each iteration issues the same loads and waits for exactly its own.
+#ifdef TRITEIA_HIP_TIMELINE
+    const long long ts_rows = wall_clock64();
+#endif
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) load_x(ring[j], wave + j * KW);
+    for (int st = wave; st < n_steps; st += DEPTH * KW) {
+#pragma unroll
+      for (int j = 0; j < DEPTH; j++) {
+        const int cur = st + j * KW;
+        if (cur < n_steps) compute_step(ring[j], cur);
+        load_w(ring[j], cur + DEPTH * KW);
+        load_x(ring[j], cur + DEPTH * KW);
+      }
     }
 
+#ifdef TRITEIA_HIP_TIMELINE
+    const long long ts_loop = wall_clock64();
+#endif
     // cross-wave reduction + epilogue, one 16-token tile at a time
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
       if (nt * 16 >= cnt) break;
-      if (nt > 0) __syncthreads();
+      if (nt > 0) lds_barrier();
       float* dst = &red[wave][r][32 * q];   // D: lane (n = r, qq = q) owns features 32q + 8j + c
 #pragma unroll
       for (int j = 0; j < 4; j++) {
@@ -257,7 +306,7 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
         *reinterpret_cast<float4_t*>(dst + 8 * j) = lo;
         *reinterpret_cast<float4_t*>(dst + 8 * j + 4) = hi;
       }
-      __syncthreads();
+      lds_barrier();
       // 16 tokens x 128 features = 256 chunks of 8 features
       for (int ch = tid; ch < 256; ch += 64 * KW) {
         const int tok = ch >> 4;
@@ -288,6 +337,14 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
         *reinterpret_cast<half8_t*>(op) = o;
       }
     }
+    // the next pass over this group's tokens reuses s_rows / red
+    if (t0 + gridDim.y * 16 * NT < count) lds_barrier();
+#ifdef TRITEIA_HIP_TIMELINE
+    if (p.timeline && lane == 0 && blockIdx.y == 0) {
+      long long* t = p.timeline + ((long)unit * KW + wave) * 4;
+      t[0] = ts_entry; t[1] = ts_rows; t[2] = ts_loop; t[3] = wall_clock64();
+    }
+#endif
   }
 }
 

@@ -66,26 +66,31 @@ int pick_nt(long tokens_per_group_hint) {
   return 4;
 }
 
-template <int NT>
-void launch_nt(const Sparse24Args& a, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((sparse24_grouped_kernel<NT, 4>), grid, dim3(256), 0, st, a);
+template <int NT, int KW, int DEPTH>
+void launch_one(const Sparse24Args& a, dim3 grid, hipStream_t st) {
+  hipLaunchKernelGGL((sparse24_grouped_kernel<NT, KW, DEPTH>), grid, dim3(64 * KW), 0, st, a);
 }
 
 int launch_sparse24(Sparse24Args a, long tokens_per_group_hint, long max_group_tokens, hipStream_t st) {
+  (void)max_group_tokens;
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   const int nt = pick_nt(tokens_per_group_hint);
-  long tsplit = (max_group_tokens + 16 * nt - 1) / (16 * nt);
+  // workgroups along y share a group's tokens 16*nt at a time; sized for the expected group
+  long tsplit = (tokens_per_group_hint + 16 * nt - 1) / (16 * nt);
   if (tsplit < 1) tsplit = 1;
   if (tsplit > 8) tsplit = 8;
   const long units = (long)a.n_groups * (a.m / 128);
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   const dim3 grid((unsigned)units, (unsigned)tsplit);
-  switch (nt) {
-    case 1: launch_nt<1>(a, grid, st); break;
-    case 2: launch_nt<2>(a, grid, st); break;
-    default: launch_nt<4>(a, grid, st); break;
-  }
-  return check_launch("sparse24_grouped_kernel");
+  const int kw = env_int("TRITEIA_HIP_KW", 4);
+  // register budget: two steps in flight for the narrow tiles, one for the 64-token tile
+  const int depth = env_int("TRITEIA_HIP_DEPTH", nt == 4 ? 1 : 2);
+#define TRY(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
+  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 1) TRY(1, 8, 2) TRY(1, 8, 3) TRY(1, 2, 2) TRY(1, 2, 4)
+  TRY(2, 4, 1) TRY(2, 4, 2) TRY(2, 8, 1)
+  TRY(4, 4, 1) TRY(4, 8, 1)
+#undef TRY
+  return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "no kernel variant for NT=%d KW=%d DEPTH=%d", nt, kw, depth);
 }
 
 void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
@@ -108,6 +113,10 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.uniform_count = 0;
   a.delta_step = 0;
   a.accumulate = 0;
+  a.xcd_swizzle = env_int("TRITEIA_HIP_XCD_SWIZZLE", 1);
+#ifdef TRITEIA_HIP_TIMELINE
+  a.timeline = reinterpret_cast<long long*>(strtoull(getenv("TRITEIA_HIP_TIMELINE_PTR") ? getenv("TRITEIA_HIP_TIMELINE_PTR") : "0", nullptr, 0));
+#endif
 }
 
 }  // namespace
