@@ -44,6 +44,8 @@ def parse():
     p.add_argument("--no-graph", action="store_true", help="time eager launches instead of one captured HIP graph")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--warm-cache", action="store_true", help="do not rotate weight copies (Infinity-Cache-warm number)")
+    p.add_argument("--calibrate-copy", action="store_true",
+                   help="also run one plain 256 MiB device copy (a known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     return p.parse_args()
 
 
@@ -187,6 +189,13 @@ def main():
         copies = max(1, min(64, int(np.ceil(1.5 * 2 ** 30 / max(touched, 1))), int(12 * 2 ** 30 // (wl.n_deltas * wl.delta_bytes)) or 1))
     prob = Problem(wl, copies, torch, ffi)
     torch.cuda.synchronize()
+    if a.calibrate_copy:
+        src = torch.empty(256 * 2 ** 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- whole-job timing: W warm-up steps, then exactly K steps
     for i in range(a.warmup):
