@@ -105,12 +105,18 @@ TRITEIA_HIP_API int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, co
                                 void* stream);
 TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n_deltas);
 
-/* Only the routing step of the call above: fills `workspace` with
- * [n_groups, n_routed, 0, 0 | g_delta[G] | g_start[G] | g_count[G] | perm[prob_n]]
- * (int32, G = min(prob_n, n_deltas)).  Exposed so that the LoRA path can share
- * one routing pass with the delta path. */
+/* Only the routing step of the call above: fills `workspace` (16-byte aligned) with
+ *   int32 header[4] = {tiles, routed tokens, deltas in use, tile size}
+ *   int32 tiles[max_tiles][4] = {delta, start, count, 0}: at most `tile size` tokens of one
+ *         delta, listed at perm[start .. start+count); a delta's tiles are adjacent
+ *   int32 perm[prob_n] = token rows grouped by delta, original order kept (stable)
+ * with max_tiles = min(prob_n, n_deltas) + prob_n / 16.  The tile size is
+ * triteia_hip_plan_tile_tokens(prob_n, n_deltas).  Exposed so that one routing pass can
+ * serve every layer of a forward pass and the LoRA path. */
 TRITEIA_HIP_API int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
                            size_t workspace_bytes, int dev, void* stream);
+
+TRITEIA_HIP_API int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas);
 
 /* The multiply step alone, on a plan made by triteia_hip_route_plan for the same
  * (prob_n, n_deltas): C[t] (+)= A[t] @ dequant(B[d]) for every routed token.  One

@@ -59,8 +59,11 @@ def test_other_argument_errors():
     assert lib.triteia_hip_bgmv(null, null, null, null, 4, 4096, 16, 1, 3, 1.0, 0, null) == _ffi.ERR_PROB_SHAPE
     # routed sbmm: workspace too small, too many deltas
     need = lib.triteia_hip_sbmm_routed_workspace_bytes(64, 16)
-    assert need == 4 * (4 + 3 * 16 + 64)
-    one = ctypes.c_void_p(1)
+    assert need == 4 * (4 + 4 * (16 + 64 // 16) + 64)
+    assert lib.triteia_hip_plan_tile_tokens(8, 8) == 16
+    assert lib.triteia_hip_plan_tile_tokens(64, 16) == 32
+    assert lib.triteia_hip_plan_tile_tokens(4096, 4) == 64
+    one = ctypes.c_void_p(16)
     assert lib.triteia_hip_route_plan(one, 0, 16, 64, one, need - 1, 0, null) == _ffi.ERR_ARGUMENT
     assert lib.triteia_hip_route_plan(one, 0, 100000, 64, one, 1 << 30, 0, null) == _ffi.ERR_KERN_SHAPE
     assert lib.triteia_hip_sgmv_tmp_size(7) == 420

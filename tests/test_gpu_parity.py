@@ -198,27 +198,30 @@ def test_sbmm_with_base_weight_accumulates_in_place(ops):
 
 
 def test_route_plan_is_a_stable_grouping():
-    from triteia_amd.python.capi import route_plan
+    from triteia_amd.python.capi import _ffi, route_plan
     say("route plan")
     rng = np.random.default_rng(51)
-    for T, N, off in [(1, 1, 0), (64, 16, 0), (200, 7, 0), (1000, 300, 0), (130, 5, 3), (70, 100, 0)]:
+    for T, N, off in [(1, 1, 0), (64, 16, 0), (200, 7, 0), (1000, 300, 0), (130, 5, 3), (70, 100, 0), (700, 3, 0)]:
         idx = rng.integers(-1, N + off, size=T).astype(np.int32)
         plan = route_plan(torch.from_numpy(idx).to(DEV), N, index_offset=off).cpu().numpy()
         d = idx - off
         valid = (d >= 0) & (d < N)
-        G = min(T, N)
-        n_groups, n_routed = plan[0], plan[1]
-        g_delta, g_start, g_count = plan[4:4 + G], plan[4 + G:4 + 2 * G], plan[4 + 2 * G:4 + 3 * G]
-        perm = plan[4 + 3 * G:4 + 3 * G + T]
+        tile = _ffi.lib().triteia_hip_plan_tile_tokens(T, N)
+        max_tiles = min(T, N) + T // 16
+        n_tiles, n_routed, n_used, tile_dev = plan[0], plan[1], plan[2], plan[3]
+        tiles = plan[4:4 + 4 * max_tiles].reshape(max_tiles, 4)[:n_tiles]
+        perm = plan[4 + 4 * max_tiles:4 + 4 * max_tiles + T]
         used = np.unique(d[valid])
-        assert n_groups == len(used) and n_routed == valid.sum()
-        assert np.array_equal(g_delta[:n_groups], used)
-        pos = 0
-        for j in range(n_groups):
-            rows = np.nonzero(d == g_delta[j])[0]          # ascending = original order
-            assert g_start[j] == pos and g_count[j] == len(rows)
+        assert tile_dev == tile and n_used == len(used) and n_routed == valid.sum()
+        pos, ti = 0, 0
+        for delta in used:
+            rows = np.nonzero(d == delta)[0]                # ascending = original order
             assert np.array_equal(perm[pos:pos + len(rows)], rows)
+            for first in range(0, len(rows), tile):          # the delta's tiles, in order, adjacent
+                assert list(tiles[ti]) == [delta, pos + first, min(tile, len(rows) - first), 0]
+                ti += 1
             pos += len(rows)
+        assert ti == n_tiles
 
 
 # ------------------------------------------------------------- lora / ldmm

@@ -91,11 +91,9 @@ struct SgmvArgs {
   long w_stride;
   long layer_off;
   // groups: indptr `seg` (group g = rows seg[g]..seg[g+1], adapter g), or the
-  // routing plan's (g_delta, g_start, g_count, perm)
+  // routing plan's tile list {adapter, start, count, 0} + perm
   const int* seg;
-  const int* g_delta;
-  const int* g_start;
-  const int* g_count;
+  const int4* tiles;
   const int* perm;
   const int* n_groups_dev;
   int n_groups;
@@ -117,9 +115,10 @@ __device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* 
     out->start = a.seg[g];
     out->count = a.seg[g + 1] - a.seg[g];
   } else {
-    adapter = a.g_delta[g];
-    out->start = a.g_start[g];
-    out->count = a.g_count[g];
+    const int4 d = a.tiles[g];
+    adapter = d.x;
+    out->start = d.y;
+    out->count = d.z;
   }
   if (out->count <= 0 || adapter < 0 || adapter >= a.n_adapters) return false;
   const _Float16* base = a.w_ptrs ? reinterpret_cast<const _Float16*>(a.w_ptrs[adapter]) : a.w_base + adapter * a.w_stride;

@@ -7,11 +7,13 @@
 // indices in any order with -1 (no delta) anywhere.
 //
 // Output (all int32, in the caller's workspace):
-//   header[0] = number of groups G (deltas that have at least one token)
-//   header[1] = number of routed tokens
-//   g_delta[G], g_start[G], g_count[G] : per group, ascending delta id
-//   perm[routed] : token rows, grouped by delta, original order kept inside a
-//                  group (stable), g_start indexes into it
+//   header[0] = number of tiles, header[1] = number of routed tokens,
+//   header[2] = number of deltas that have at least one token, header[3] = tile size
+//   tiles[..] = {delta, start, count, 0}: `count` <= tile size tokens of one delta,
+//               listed at perm[start .. start+count); ascending delta id, a delta's
+//               tiles are adjacent
+//   perm[routed] = token rows, grouped by delta, original order kept inside a
+//               delta (stable)
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -21,21 +23,29 @@ namespace triteia_hip {
 constexpr int kPlanHeaderInts = 4;
 constexpr int kPlanMaxDeltas = 8192;  // per-delta cursors live in LDS
 constexpr int kPlanThreads = 256;
+constexpr int kPlanMinTile = 16;      // smallest tile size a plan can be built for
 
 struct PlanLayout {
-  int header, g_delta, g_start, g_count, perm, total;  // offsets in ints
+  int header, tiles, perm, total;  // offsets in ints
+  int max_tiles;
 };
 
+// The layout depends only on (tokens, deltas), not on the tile size the plan is built
+// for, so that every consumer finds `perm` without knowing it.
 __host__ __device__ inline PlanLayout plan_layout(int n_tokens, int n_deltas) {
   const int g = n_deltas < n_tokens ? n_deltas : n_tokens;
   PlanLayout l;
+  l.max_tiles = g + n_tokens / kPlanMinTile;
   l.header = 0;
-  l.g_delta = kPlanHeaderInts;
-  l.g_start = l.g_delta + g;
-  l.g_count = l.g_start + g;
-  l.perm = l.g_count + g;
+  l.tiles = kPlanHeaderInts;
+  l.perm = l.tiles + 4 * l.max_tiles;
   l.total = l.perm + n_tokens;
   return l;
+}
+
+__host__ __device__ inline int plan_max_tiles(int n_tokens, int n_deltas, int tile) {
+  const int g = n_deltas < n_tokens ? n_deltas : n_tokens;
+  return g + n_tokens / tile;
 }
 
 __device__ __forceinline__ int wave_excl_scan(int v, int lane, int* total) {
@@ -49,9 +59,10 @@ __device__ __forceinline__ int wave_excl_scan(int v, int lane, int* total) {
   return incl - v;
 }
 
-// One workgroup.  indices[t] outside [0, n_deltas) means "no delta".
+// One workgroup.  indices[t] - index_offset outside [0, n_deltas) means "no delta".
 __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __restrict__ indices, int n_tokens,
-                                                                 int n_deltas, int index_offset, int* __restrict__ ws) {
+                                                                 int n_deltas, int index_offset, int tile,
+                                                                 int* __restrict__ ws) {
   __shared__ int s_cursor[kPlanMaxDeltas];
   const PlanLayout L = plan_layout(n_tokens, n_deltas);
   const int tid = threadIdx.x;
@@ -66,30 +77,31 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
   __syncthreads();
 
   if (tid < 64) {
-    // exclusive scan of the counts (-> first slot of every delta) and compaction
-    // of the deltas that have tokens, 64 deltas per iteration
-    int running = 0, groups = 0;
+    // exclusive scans over the deltas, 64 per iteration: token counts -> first slot in perm,
+    // tile counts -> first tile
+    int running = 0, tiles = 0, groups = 0;
+    int4* tile_out = reinterpret_cast<int4*>(ws + L.tiles);
     for (int base = 0; base < n_deltas; base += 64) {
       const int d = base + lane;
       const int c = d < n_deltas ? s_cursor[d] : 0;
-      int chunk_total;
-      const int offs = running + wave_excl_scan(c, lane, &chunk_total);
-      const unsigned long long act = __ballot(c > 0);
-      if (c > 0) {
-        const int pos = groups + __popcll(act & ((1ull << lane) - 1ull));
-        ws[L.g_delta + pos] = d;
-        ws[L.g_start + pos] = offs;
-        ws[L.g_count + pos] = c;
+      int chunk_tokens, chunk_tiles;
+      const int offs = running + wave_excl_scan(c, lane, &chunk_tokens);
+      const int nt = (c + tile - 1) / tile;
+      const int tpos = tiles + wave_excl_scan(nt, lane, &chunk_tiles);
+      for (int i = 0; i < nt; i++) {
+        const int first = i * tile;
+        tile_out[tpos + i] = make_int4(d, offs + first, min(tile, c - first), 0);
       }
       if (d < n_deltas) s_cursor[d] = offs;
-      running += chunk_total;
-      groups += __popcll(act);
+      running += chunk_tokens;
+      tiles += chunk_tiles;
+      groups += __popcll(__ballot(c > 0));
     }
     if (lane == 0) {
-      ws[L.header + 0] = groups;
+      ws[L.header + 0] = tiles;
       ws[L.header + 1] = running;
-      ws[L.header + 2] = 0;
-      ws[L.header + 3] = 0;
+      ws[L.header + 2] = groups;
+      ws[L.header + 3] = tile;
     }
     // stable placement: 64 tokens at a time, tokens with equal delta ranked by lane order
     for (int base = 0; base < n_tokens; base += 64) {

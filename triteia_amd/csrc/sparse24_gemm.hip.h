@@ -62,8 +62,11 @@ struct Sparse24Args {
   long out_stride;          // elements between rows
   int m;                    // output features
   int k;                    // input features
-  // groups: explicit arrays, or (if g_delta == nullptr) group j = delta
-  // j*delta_step with rows [j*uniform_count, (j+1)*uniform_count)
+  // groups, one of three forms:
+  //   tiles   : packed {delta, start, count, 0} per group (the routing plan's tile list)
+  //   g_*     : three separate arrays (the reference's run table)
+  //   neither : group j = delta j*delta_step with rows [j*uniform_count, (j+1)*uniform_count)
+  const int4* tiles;
   const int* g_delta;
   const int* g_start;
   const int* g_count;
@@ -113,6 +116,196 @@ struct StepFrag {
 
 constexpr int kRedStride = 132;  // floats per token row in the reduction buffer (128 + pad)
 
+// Everything one workgroup knows about its (group, column block) before touching tokens.
+struct TileCtx {
+  const uint4_t* qw_lane;   // this lane's first weight vector in packed row 0
+  const uint4_t* mt_lane;   // this lane's first metadata vector in packed row 0
+  const _Float16* sc;       // scales of the 128 columns
+  long qrow, mrow;          // vectors per packed row (weights, metadata)
+  int k_rows, n_steps;      // packed rows, 128-k steps
+  int cb;                   // column block
+  int tid, wave, lane, r, q;
+};
+
+// One pass over K for up to 16*NTT tokens of one group: loads, sparse MFMAs, cross-wave
+// reduction, scaled fp16 store.  `first` = index of the pass's first token in the group's list.
+template <int NTT, int KW, int DEPTH>
+__device__ __forceinline__ void tile_pass(const Sparse24Args& p, const TileCtx& c, int first, int cnt,
+                                          float (*red)[16][kRedStride], int* s_rows) {
+  const int r = c.r, q = c.q, wave = c.wave;
+  const int k_rows = c.k_rows, n_steps = c.n_steps;
+
+  // Steps past the end of K (st >= n_steps) read step 0 again: cheap cache hits that keep the
+  // load count per iteration constant; they are never multiplied.
+  auto load_w = [&](StepFrag<NTT>& f, int st) {
+    const int tr0 = (st < n_steps ? st : 0) << 2;
+    const int tr = min(tr0 + q, k_rows - 1);  // clamped: rows past the end are cancelled by zero B
+    const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
+    const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
+#pragma unroll
+    for (int a = 0; a < 4; a++) f.wq[a] = wp[a];
+    f.mt[0] = mp[0];
+    f.mt[1] = mp[8];
+  };
+
+  // Start-up order matters (vector loads return in order): first the tiny per-lane read of
+  // this lane's token rows, then the weight stream (which only needs the delta id), and the
+  // activation loads once the rows have arrived.  No barrier is needed before the K loop.
+  int rows[NTT];
+#pragma unroll
+  for (int nt = 0; nt < NTT; nt++) {
+    const int slot = min(nt * 16 + r, cnt - 1);   // slots past the end re-read the last row
+    rows[nt] = p.perm ? p.perm[first + slot] : first + slot;
+  }
+  StepFrag<NTT> ring[DEPTH];
+#pragma unroll
+  for (int j = 0; j < DEPTH; j++) load_w(ring[j], wave + j * KW);
+
+  // Every lane always loads from a valid address, so that the number of loads per step is
+  // fixed and the hardware load counter can be waited on exactly (the output columns of the
+  // duplicated slots are never stored).
+  const _Float16* xrow[NTT];
+#pragma unroll
+  for (int nt = 0; nt < NTT; nt++) {
+    // B operand slot layout: this lane supplies k offsets 8*(q%2) + {0..7} of
+    // packed rows tr0 + q/2 and tr0 + 2 + q/2
+    xrow[nt] = p.x + (long)rows[nt] * p.x_stride + 32 * (q >> 1) + 8 * (q & 1);
+  }
+  if (wave == 0 && q == 0) {
+#pragma unroll
+    for (int nt = 0; nt < NTT; nt++) s_rows[nt * 16 + r] = (nt * 16 + r < cnt) ? rows[nt] : -1;
+  }
+
+  float4_t acc[8][NTT];
+#pragma unroll
+  for (int cc = 0; cc < 8; cc++)
+#pragma unroll
+    for (int nt = 0; nt < NTT; nt++) acc[cc][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  auto load_x = [&](StepFrag<NTT>& f, int st) {
+    const int tr0 = (st < n_steps ? st : 0) << 2;
+    // rows tr0+2.. may lie past the end of K in the last step: clamp the address, zero at use
+    const long xoff_a = (long)min(tr0, k_rows - 1 - (q >> 1)) * 32;
+    const long xoff_b = (long)min(tr0 + 2, k_rows - 1 - (q >> 1)) * 32;
+#pragma unroll
+    for (int nt = 0; nt < NTT; nt++) {
+      f.xa[nt][0] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_a);
+      f.xa[nt][1] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_a + 16);
+      f.xb[nt][0] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_b);
+      f.xb[nt][1] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_b + 16);
+    }
+  };
+
+  auto compute_step = [&](const StepFrag<NTT>& f, int st) {
+    const int tr0 = st << 2;
+    const bool tail = tr0 + 4 > k_rows;            // wave-uniform: only the last, partial step
+    const bool ok_a = (tr0 + (q >> 1)) < k_rows;
+    const bool ok_b = (tr0 + 2 + (q >> 1)) < k_rows;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      half16_t b[NTT];
+#pragma unroll
+      for (int nt = 0; nt < NTT; nt++) {
+        typedef uint32_t uint8_t_v __attribute__((ext_vector_type(8)));
+        uint8_t_v bb = {f.xa[nt][u][0], f.xa[nt][u][1], f.xa[nt][u][2], f.xa[nt][u][3],
+                        f.xb[nt][u][0], f.xb[nt][u][1], f.xb[nt][u][2], f.xb[nt][u][3]};
+        if (tail) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            if (!ok_a) bb[i] = 0u;
+            if (!ok_b) bb[4 + i] = 0u;
+          }
+        }
+        b[nt] = __builtin_bit_cast(half16_t, bb);
+      }
+#pragma unroll
+      for (int cc = 0; cc < 8; cc++) {
+        const int w = cc & 3;         // word inside each weight vector
+        const int b2 = cc >> 2;       // upper / lower 4 columns of the 8-column block
+        uint4_t av;
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+          uint32_t word = f.wq[a][w];
+          if (b2) word >>= 8;
+          av[a] = u ? dequant_odd(word) : dequant_even(word);
+        }
+        const half8_t A = __builtin_bit_cast(half8_t, av);
+        const int idx = (int)f.mt[(cc >> 1) & 1][(cc & 1) * 2 + u];
+#pragma unroll
+        for (int nt = 0; nt < NTT; nt++) {
+          if (b2)
+            acc[cc][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A, b[nt], acc[cc][nt], idx, 0, 1);
+          else
+            acc[cc][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A, b[nt], acc[cc][nt], idx, 0, 0);
+        }
+      }
+    }
+  };
+
+  // K loop: wave w takes steps w, w + KW, ...; DEPTH steps of loads are kept in flight in
+  // registers (ring of fragments, statically indexed through the unrolled inner loop).
+  // The body is branch-free apart from the wave-uniform "is this step real" test around the
+  // arithmetic, so each iteration issues the same loads and waits for exactly its own.
+#pragma unroll
+  for (int j = 0; j < DEPTH; j++) load_x(ring[j], wave + j * KW);
+  for (int st = wave; st < n_steps; st += DEPTH * KW) {
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) {
+      const int cur = st + j * KW;
+      if (cur < n_steps) compute_step(ring[j], cur);
+      load_w(ring[j], cur + DEPTH * KW);
+      load_x(ring[j], cur + DEPTH * KW);
+    }
+  }
+
+  // cross-wave reduction + epilogue, one 16-token tile at a time
+#pragma unroll
+  for (int nt = 0; nt < NTT; nt++) {
+    if (nt * 16 >= cnt) break;
+    if (nt > 0) lds_barrier();
+    float* dst = &red[wave][r][32 * q];   // D: lane (n = r, qq = q) owns features 32q + 8j + c
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      float4_t lo = {acc[0][nt][j], acc[1][nt][j], acc[2][nt][j], acc[3][nt][j]};
+      float4_t hi = {acc[4][nt][j], acc[5][nt][j], acc[6][nt][j], acc[7][nt][j]};
+      *reinterpret_cast<float4_t*>(dst + 8 * j) = lo;
+      *reinterpret_cast<float4_t*>(dst + 8 * j + 4) = hi;
+    }
+    lds_barrier();
+    // 16 tokens x 128 features = 256 chunks of 8 features
+    for (int ch = c.tid; ch < 256; ch += 64 * KW) {
+      const int tok = ch >> 4;
+      const int f0 = (ch & 15) * 8;
+      const int row = s_rows[nt * 16 + tok];
+      if (row < 0) continue;
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = 0.f;
+#pragma unroll
+      for (int w = 0; w < KW; w++) {
+        const float4_t a0 = *reinterpret_cast<const float4_t*>(&red[w][tok][f0]);
+        const float4_t a1 = *reinterpret_cast<const float4_t*>(&red[w][tok][f0 + 4]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) { v[i] += a0[i]; v[4 + i] += a1[i]; }
+      }
+      const half8_t sv = *reinterpret_cast<const half8_t*>(c.sc + f0);
+      _Float16* op = p.out + (long)row * p.out_stride + c.cb * 128 + f0;
+      half8_t o;
+      if (p.accumulate) {
+        const half8_t old = *reinterpret_cast<const half8_t*>(op);
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = (_Float16)((float)old[i] + v[i] * (float)sv[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = (_Float16)(v[i] * (float)sv[i]);
+      }
+      *reinterpret_cast<half8_t*>(op) = o;
+    }
+  }
+}
+
+// NT = widest token tile (16*NT tokens per pass) the instantiation supports; narrower passes
+// take the cheaper code path (fewer activation loads and MFMAs) at the same register budget.
 template <int NT, int KW, int DEPTH>
 __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse24Args p) {
   __shared__ float red[KW][16][kRedStride];
@@ -131,7 +324,12 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
   // group descriptor and live group count are fetched side by side (no dependent chain);
   // grp < p.n_groups (the host's upper bound) keeps the descriptor reads in bounds
   int delta, start, count;
-  if (p.g_delta) {
+  if (p.tiles) {
+    const int4 d = p.tiles[grp];
+    delta = d.x;
+    start = d.y;
+    count = d.z;
+  } else if (p.g_delta) {
     delta = p.g_delta[grp];
     start = p.g_start[grp];
     count = p.g_count[grp];
@@ -144,208 +342,40 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
   if (grp >= n_groups) return;
   if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
 
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6;
-  const int lane = tid & 63;
-  const int r = lane & 15;
-  const int q = lane >> 4;
-
-  const int k_rows = p.k >> 5;                 // packed rows (32 dense k each)
-  const int n_steps = (k_rows + 3) >> 2;       // 128 dense k per step
-  const long qrow = p.m >> 1;                  // vectors per packed weight row
-  const long mrow = p.m >> 2;                  // vectors per packed metadata row
-
-  const uint4_t* qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * r;
-  const uint4_t* mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (r >> 3)) * 16 + (r & 7);
-  const _Float16* sc = p.scales + (long)delta * p.scales_stride + cb * 128;
-
-  // Steps past the end of K (st >= n_steps) read step 0 again: cheap cache hits that keep the
-  // load count per iteration constant; they are never multiplied.
-  auto load_w = [&](StepFrag<NT>& f, int st) {
-    const int tr0 = (st < n_steps ? st : 0) << 2;
-    const int tr = min(tr0 + q, k_rows - 1);  // clamped: rows past the end are cancelled by zero B
-    const uint4_t* wp = qw_lane + (long)tr * qrow;
-    const uint4_t* mp = mt_lane + (long)tr * mrow;
-#pragma unroll
-    for (int a = 0; a < 4; a++) f.wq[a] = wp[a];
-    f.mt[0] = mp[0];
-    f.mt[1] = mp[8];
-  };
+  TileCtx c;
+  c.tid = threadIdx.x;
+  c.wave = c.tid >> 6;
+  c.lane = c.tid & 63;
+  c.r = c.lane & 15;
+  c.q = c.lane >> 4;
+  c.cb = cb;
+  c.k_rows = p.k >> 5;                 // packed rows (32 dense k each)
+  c.n_steps = (c.k_rows + 3) >> 2;     // 128 dense k per step
+  c.qrow = p.m >> 1;
+  c.mrow = p.m >> 2;
+  c.qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * c.r;
+  c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.r >> 3)) * 16 + (c.r & 7);
+  c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;
 
   // blockIdx.y splits a group's tokens between workgroups (each re-streams the weights)
   for (int t0 = blockIdx.y * 16 * NT; t0 < count; t0 += gridDim.y * 16 * NT) {
     const int cnt = min(count - t0, 16 * NT);
-    // Start-up order matters (vector loads return in order): first the tiny per-lane read of
-    // this lane's token rows, then the weight stream (which only needs the delta id), and the
-    // activation loads once the rows have arrived.  No barrier is needed before the K loop.
-    int rows[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      const int slot = min(nt * 16 + r, cnt - 1);   // slots past the end re-read the last row
-      rows[nt] = p.perm ? p.perm[start + t0 + slot] : start + t0 + slot;
-    }
-    StepFrag<NT> ring[DEPTH];
-#pragma unroll
-    for (int j = 0; j < DEPTH; j++) load_w(ring[j], wave + j * KW);
-
-    // Every lane always loads from a valid address, so that the number of loads per step is
-    // fixed and the hardware load counter can be waited on exactly (the output columns of the
-    // duplicated slots are never stored).
-    const _Float16* xrow[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      // B operand slot layout: this lane supplies k offsets 8*(q%2) + {0..7} of
-      // packed rows tr0 + q/2 and tr0 + 2 + q/2
-      xrow[nt] = p.x + (long)rows[nt] * p.x_stride + 32 * (q >> 1) + 8 * (q & 1);
-    }
-    if (wave == 0 && q == 0) {
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++) s_rows[nt * 16 + r] = (nt * 16 + r < cnt) ? rows[nt] : -1;
-    }
-
-    float4_t acc[8][NT];
-#pragma unroll
-    for (int c = 0; c < 8; c++)
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++) acc[c][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-    auto load_x = [&](StepFrag<NT>& f, int st) {
-      const int tr0 = (st < n_steps ? st : 0) << 2;
-      // rows tr0+2.. may lie past the end of K in the last step: clamp the address, zero at use
-      const long xoff_a = (long)min(tr0, k_rows - 1 - (q >> 1)) * 32;
-      const long xoff_b = (long)min(tr0 + 2, k_rows - 1 - (q >> 1)) * 32;
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        f.xa[nt][0] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_a);
-        f.xa[nt][1] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_a + 16);
-        f.xb[nt][0] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_b);
-        f.xb[nt][1] = *reinterpret_cast<const uint4_t*>(xrow[nt] + xoff_b + 16);
-      }
-    };
-
-    auto compute_step = [&](const StepFrag<NT>& f, int st) {
-      const int tr0 = st << 2;
-      const bool tail = tr0 + 4 > k_rows;            // wave-uniform: only the last, partial step
-      const bool ok_a = (tr0 + (q >> 1)) < k_rows;
-      const bool ok_b = (tr0 + 2 + (q >> 1)) < k_rows;
-#pragma unroll
-      for (int u = 0; u < 2; u++) {
-        half16_t b[NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-          typedef uint32_t uint8_t_v __attribute__((ext_vector_type(8)));
-          uint8_t_v bb = {f.xa[nt][u][0], f.xa[nt][u][1], f.xa[nt][u][2], f.xa[nt][u][3],
-                          f.xb[nt][u][0], f.xb[nt][u][1], f.xb[nt][u][2], f.xb[nt][u][3]};
-          if (tail) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-              if (!ok_a) bb[i] = 0u;
-              if (!ok_b) bb[4 + i] = 0u;
-            }
-          }
-          b[nt] = __builtin_bit_cast(half16_t, bb);
-        }
-#pragma unroll
-        for (int c = 0; c < 8; c++) {
-          const int w = c & 3;         // word inside each weight vector
-          const int b2 = c >> 2;       // upper / lower 4 columns of the 8-column block
-          uint4_t av;
-#pragma unroll
-          for (int a = 0; a < 4; a++) {
-            uint32_t word = f.wq[a][w];
-            if (b2) word >>= 8;
-            av[a] = u ? dequant_odd(word) : dequant_even(word);
-          }
-          const half8_t A = __builtin_bit_cast(half8_t, av);
-          const int idx = (int)f.mt[(c >> 1) & 1][(c & 1) * 2 + u];
-#pragma unroll
-          for (int nt = 0; nt < NT; nt++) {
-            if (nt * 16 < cnt) {
-              if (b2)
-                acc[c][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A, b[nt], acc[c][nt], idx, 0, 1);
-              else
-                acc[c][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A, b[nt], acc[c][nt], idx, 0, 0);
-            }
-          }
-        }
-      }
-    };
-
-    // K loop: wave w takes steps w, w + KW, ...; DEPTH steps of loads are kept in flight in
-    // registers (ring of fragments, statically indexed through the unrolled inner loop).
-    // The body is branch-free apart from the wave-uniform "is this step real" test around the
-    // arithmetic, so each iteration issues the same loads and waits for exactly its own.
-#ifdef TRITEIA_HIP_TIMELINE
-    const long long ts_rows = wall_clock64();
-#endif
-#pragma unroll
-    for (int j = 0; j < DEPTH; j++) load_x(ring[j], wave + j * KW);
-    for (int st = wave; st < n_steps; st += DEPTH * KW) {
-#pragma unroll
-      for (int j = 0; j < DEPTH; j++) {
-        const int cur = st + j * KW;
-        if (cur < n_steps) compute_step(ring[j], cur);
-        load_w(ring[j], cur + DEPTH * KW);
-        load_x(ring[j], cur + DEPTH * KW);
-      }
-    }
-
-#ifdef TRITEIA_HIP_TIMELINE
-    const long long ts_loop = wall_clock64();
-#endif
-    // cross-wave reduction + epilogue, one 16-token tile at a time
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      if (nt * 16 >= cnt) break;
-      if (nt > 0) lds_barrier();
-      float* dst = &red[wave][r][32 * q];   // D: lane (n = r, qq = q) owns features 32q + 8j + c
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        float4_t lo = {acc[0][nt][j], acc[1][nt][j], acc[2][nt][j], acc[3][nt][j]};
-        float4_t hi = {acc[4][nt][j], acc[5][nt][j], acc[6][nt][j], acc[7][nt][j]};
-        *reinterpret_cast<float4_t*>(dst + 8 * j) = lo;
-        *reinterpret_cast<float4_t*>(dst + 8 * j + 4) = hi;
-      }
-      lds_barrier();
-      // 16 tokens x 128 features = 256 chunks of 8 features
-      for (int ch = tid; ch < 256; ch += 64 * KW) {
-        const int tok = ch >> 4;
-        const int f0 = (ch & 15) * 8;
-        const int row = s_rows[nt * 16 + tok];
-        if (row < 0) continue;
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = 0.f;
-#pragma unroll
-        for (int w = 0; w < KW; w++) {
-          const float4_t a0 = *reinterpret_cast<const float4_t*>(&red[w][tok][f0]);
-          const float4_t a1 = *reinterpret_cast<const float4_t*>(&red[w][tok][f0 + 4]);
-#pragma unroll
-          for (int i = 0; i < 4; i++) { v[i] += a0[i]; v[4 + i] += a1[i]; }
-        }
-        const half8_t sv = *reinterpret_cast<const half8_t*>(sc + f0);
-        _Float16* op = p.out + (long)row * p.out_stride + cb * 128 + f0;
-        half8_t o;
-        if (p.accumulate) {
-          const half8_t old = *reinterpret_cast<const half8_t*>(op);
-#pragma unroll
-          for (int i = 0; i < 8; i++) o[i] = (_Float16)((float)old[i] + v[i] * (float)sv[i]);
-        } else {
-#pragma unroll
-          for (int i = 0; i < 8; i++) o[i] = (_Float16)(v[i] * (float)sv[i]);
-        }
-        *reinterpret_cast<half8_t*>(op) = o;
-      }
+    if (NT == 1 || cnt <= 16) {
+      tile_pass<1, KW, (NT == 1 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);
+    } else if (NT == 2 || cnt <= 32) {
+      tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);
+    } else {
+      tile_pass<NT, KW, DEPTH>(p, c, start + t0, cnt, red, s_rows);
     }
     // the next pass over this group's tokens reuses s_rows / red
     if (t0 + gridDim.y * 16 * NT < count) lds_barrier();
-#ifdef TRITEIA_HIP_TIMELINE
-    if (p.timeline && lane == 0 && blockIdx.y == 0) {
-      long long* t = p.timeline + ((long)unit * KW + wave) * 4;
-      t[0] = ts_entry; t[1] = ts_rows; t[2] = ts_loop; t[3] = wall_clock64();
-    }
-#endif
   }
+#ifdef TRITEIA_HIP_TIMELINE
+  if (p.timeline && c.lane == 0 && blockIdx.y == 0) {
+    long long* t = p.timeline + ((long)unit * KW + c.wave) * 4;
+    t[0] = ts_entry; t[1] = 0; t[2] = 0; t[3] = wall_clock64();
+  }
+#endif
 }
 
 }  // namespace triteia_hip

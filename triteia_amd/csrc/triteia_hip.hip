@@ -57,12 +57,14 @@ int check_gemm_shape(int prob_m, int prob_n, int prob_k, int groupsize) {
   return TRITEIA_HIP_OK;
 }
 
-// tokens-per-group tile of the kernel: 16 * NT rows share one pass over the weights
-int pick_nt(long tokens_per_group_hint) {
+// Token tile of the grouped kernel: 16 * NT rows share one pass over the weights.  Chosen from
+// what the host knows (tokens, groups); the routing plan cuts groups into tiles of this size.
+int pick_nt(long tokens, long groups) {
   const int forced = env_int("TRITEIA_HIP_NT", 0);
   if (forced == 1 || forced == 2 || forced == 4) return forced;
-  if (tokens_per_group_hint <= 16) return 1;
-  if (tokens_per_group_hint <= 32) return 2;
+  if (groups < 1) groups = 1;
+  if (tokens <= 16) return 1;
+  if (tokens <= 24 * groups) return 2;   // typical group well under 32 tokens
   return 4;
 }
 
@@ -71,14 +73,12 @@ void launch_one(const Sparse24Args& a, dim3 grid, hipStream_t st) {
   hipLaunchKernelGGL((sparse24_grouped_kernel<NT, KW, DEPTH>), grid, dim3(64 * KW), 0, st, a);
 }
 
-int launch_sparse24(Sparse24Args a, long tokens_per_group_hint, long max_group_tokens, hipStream_t st) {
-  (void)max_group_tokens;
+// `nt`: token tile class; `tsplit`: workgroups along y sharing one group's tokens (legacy / uniform
+// group forms only; plan tiles never exceed one pass).
+int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
-  const int nt = pick_nt(tokens_per_group_hint);
-  // workgroups along y share a group's tokens 16*nt at a time; sized for the expected group
-  long tsplit = (tokens_per_group_hint + 16 * nt - 1) / (16 * nt);
   if (tsplit < 1) tsplit = 1;
-  if (tsplit > 8) tsplit = 8;
+  if (tsplit > 65535) tsplit = 65535;
   const long units = (long)a.n_groups * (a.m / 128);
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   const dim3 grid((unsigned)units, (unsigned)tsplit);
@@ -86,9 +86,9 @@ int launch_sparse24(Sparse24Args a, long tokens_per_group_hint, long max_group_t
   // register budget: two steps in flight for the narrow tiles, one for the 64-token tile
   const int depth = env_int("TRITEIA_HIP_DEPTH", nt == 4 ? 1 : 2);
 #define TRY(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
-  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 1) TRY(1, 8, 2) TRY(1, 8, 3) TRY(1, 2, 2) TRY(1, 2, 4)
+  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 2)
   TRY(2, 4, 1) TRY(2, 4, 2) TRY(2, 8, 1)
-  TRY(4, 4, 1) TRY(4, 8, 1)
+  TRY(4, 4, 1)
 #undef TRY
   return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "no kernel variant for NT=%d KW=%d DEPTH=%d", nt, kw, depth);
 }
@@ -108,6 +108,7 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.m = prob_m;
   a.k = prob_k;
   a.n_deltas = n_deltas;
+  a.tiles = nullptr;
   a.g_delta = a.g_start = a.g_count = a.perm = a.n_groups_dev = nullptr;
   a.n_groups = 0;
   a.uniform_count = 0;
@@ -140,7 +141,8 @@ int triteia_hip_mul_2_4(const void* A, const void* B, const void* meta, void* C,
   fill_weights(a, A, B, meta, C, s, prob_m, prob_k, 1);
   a.n_groups = 1;
   a.uniform_count = prob_n;
-  return launch_sparse24(a, prob_n, prob_n, static_cast<hipStream_t>(stream));
+  const int nt = pick_nt(prob_n, 1);
+  return launch_sparse24(a, nt, (prob_n + 16 * nt - 1) / (16 * nt), static_cast<hipStream_t>(stream));
 }
 
 int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
@@ -156,7 +158,8 @@ int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, v
   a.n_groups = batch;
   a.uniform_count = tokens;
   a.delta_step = 1;
-  return launch_sparse24(a, tokens, tokens, static_cast<hipStream_t>(stream));
+  const int nt = pick_nt(tokens, 1);
+  return launch_sparse24(a, nt, (tokens + 16 * nt - 1) / (16 * nt), static_cast<hipStream_t>(stream));
 }
 
 int triteia_hip_bmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m, int prob_n,
@@ -185,13 +188,20 @@ int triteia_hip_sbmm_2_4(const void* A, const void* B, const void* meta, void* C
   a.g_start = static_cast<const int*>(starts);
   a.g_count = static_cast<const int*>(counts);
   a.n_groups = prob_r;
-  const long hint = (4L * prob_n + prob_r - 1) / prob_r;
-  return launch_sparse24(a, hint, prob_n, static_cast<hipStream_t>(stream));
+  // run lengths live on the device: size the tile and the token split for a few times the average run
+  const int nt = pick_nt(prob_n, prob_r);
+  long tsplit = (4L * prob_n / prob_r + 16 * nt - 1) / (16 * nt);
+  if (tsplit > 16) tsplit = 16;
+  return launch_sparse24(a, nt, tsplit, static_cast<hipStream_t>(stream));
 }
 
 size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n_deltas) {
   if (prob_n < 0 || n_deltas < 0) return 0;
   return sizeof(int) * (size_t)plan_layout(prob_n, n_deltas).total;
+}
+
+int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas) {
+  return 16 * pick_nt(prob_n, prob_n < n_deltas ? prob_n : n_deltas);
 }
 
 int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
@@ -202,11 +212,14 @@ int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_de
   if (!workspace || workspace_bytes < triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas))
     return fail(TRITEIA_HIP_ERR_ARGUMENT, "route_plan: workspace must hold %zu bytes (got %zu)",
                 triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas), workspace_bytes);
+  if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+    return fail(TRITEIA_HIP_ERR_ARGUMENT, "route_plan: workspace must be 16-byte aligned");
   if (prob_n > 0 && !token_indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "route_plan: null indices");
   DeviceGuard g(dev);
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   hipLaunchKernelGGL(route_plan_kernel, dim3(1), dim3(kPlanThreads), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const int*>(token_indices), prob_n, n_deltas, index_offset, static_cast<int*>(workspace));
+                     static_cast<const int*>(token_indices), prob_n, n_deltas, index_offset,
+                     triteia_hip_plan_tile_tokens(prob_n, n_deltas), static_cast<int*>(workspace));
   return check_launch("route_plan_kernel");
 }
 
@@ -222,17 +235,15 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   const PlanLayout L = plan_layout(prob_n, n_deltas);
   const int* ws = static_cast<const int*>(plan);
+  const int tile = triteia_hip_plan_tile_tokens(prob_n, n_deltas);
   Sparse24Args a;
   fill_weights(a, A, B, meta, C, s, prob_m, prob_k, n_deltas);
-  a.g_delta = ws + L.g_delta;
-  a.g_start = ws + L.g_start;
-  a.g_count = ws + L.g_count;
+  a.tiles = reinterpret_cast<const int4*>(ws + L.tiles);
   a.perm = ws + L.perm;
   a.n_groups_dev = ws + L.header;
-  a.n_groups = prob_n < n_deltas ? prob_n : n_deltas;
+  a.n_groups = plan_max_tiles(prob_n, n_deltas, tile);
   a.accumulate = accumulate;
-  const long hint = (4L * prob_n + a.n_groups - 1) / a.n_groups;
-  return launch_sparse24(a, hint, prob_n, static_cast<hipStream_t>(stream));
+  return launch_sparse24(a, tile / 16, 1, static_cast<hipStream_t>(stream));
 }
 
 int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, void* C, const void* s,
@@ -345,12 +356,10 @@ int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride
   a.d_out = d_out;
   a.w_base = static_cast<const _Float16*>(w_base);
   a.w_stride = w_stride;
-  a.g_delta = ws + L.g_delta;
-  a.g_start = ws + L.g_start;
-  a.g_count = ws + L.g_count;
+  a.tiles = reinterpret_cast<const int4*>(ws + L.tiles);
   a.perm = ws + L.perm;
   a.n_groups_dev = ws + L.header;
-  a.n_groups = prob_n < n_adapters ? prob_n : n_adapters;
+  a.n_groups = plan_max_tiles(prob_n, n_adapters, triteia_hip_plan_tile_tokens(prob_n, n_adapters));
   a.n_adapters = n_adapters;
   a.scale = scale;
   return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream));
