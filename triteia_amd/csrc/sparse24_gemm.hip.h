@@ -125,12 +125,15 @@ struct TileCtx {
   int k_rows, n_steps;      // packed rows, 128-k steps
   int cb;                   // column block
   int tid, wave, lane, r, q;
+#ifdef TRITEIA_HIP_TIMELINE
+  long long ts[4];          // debug builds: entry, operands requested, K loop done, end
+#endif
 };
 
 // One pass over K for up to 16*NTT tokens of one group: loads, sparse MFMAs, cross-wave
 // reduction, scaled fp16 store.  `first` = index of the pass's first token in the group's list.
 template <int NTT, int KW, int DEPTH>
-__device__ __forceinline__ void tile_pass(const Sparse24Args& p, const TileCtx& c, int first, int cnt,
+__device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int first, int cnt,
                                           float (*red)[16][kRedStride], int* s_rows) {
   const int r = c.r, q = c.q, wave = c.wave;
   const int k_rows = c.k_rows, n_steps = c.n_steps;
@@ -246,6 +249,9 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, const TileCtx& 
   // registers (ring of fragments, statically indexed through the unrolled inner loop).
   // The body is branch-free apart from the wave-uniform "is this step real" test around the
   // arithmetic, so each iteration issues the same loads and waits for exactly its own.
+#ifdef TRITEIA_HIP_TIMELINE
+  c.ts[1] = wall_clock64();
+#endif
 #pragma unroll
   for (int j = 0; j < DEPTH; j++) load_x(ring[j], wave + j * KW);
   for (int st = wave; st < n_steps; st += DEPTH * KW) {
@@ -258,6 +264,9 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, const TileCtx& 
     }
   }
 
+#ifdef TRITEIA_HIP_TIMELINE
+  c.ts[2] = wall_clock64();
+#endif
   // cross-wave reduction + epilogue, one 16-token tile at a time
 #pragma unroll
   for (int nt = 0; nt < NTT; nt++) {
@@ -314,13 +323,16 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
 #ifdef TRITEIA_HIP_TIMELINE
   const long long ts_entry = wall_clock64();
 #endif
+  // Unit = (group, column block).  Workgroups are dealt round-robin to the 8 XCDs (each with
+  // its own L2); the column blocks of a group are numbered so that every XCD owns a contiguous
+  // run of them: the per-group unit count is padded to a multiple of 8 (padding units exit).
   const int col_blocks = p.m >> 7;
+  const int cb_pad = (col_blocks + 7) & ~7;
   const int unit = blockIdx.x;
-  const int grp = unit / col_blocks;
-  int cb = unit - grp * col_blocks;
-  // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): give every XCD a
-  // contiguous run of column blocks instead of every 8th one.
-  if (p.xcd_swizzle && (col_blocks & 7) == 0) cb = (cb & 7) * (col_blocks >> 3) + (cb >> 3);
+  const int grp = unit / cb_pad;
+  const int i = unit - grp * cb_pad;
+  const int cb = p.xcd_swizzle ? (i & 7) * (cb_pad >> 3) + (i >> 3) : i;
+  if (cb >= col_blocks) return;
   // group descriptor and live group count are fetched side by side (no dependent chain);
   // grp < p.n_groups (the host's upper bound) keeps the descriptor reads in bounds
   int delta, start, count;
@@ -373,7 +385,7 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
 #ifdef TRITEIA_HIP_TIMELINE
   if (p.timeline && c.lane == 0 && blockIdx.y == 0) {
     long long* t = p.timeline + ((long)unit * KW + c.wave) * 4;
-    t[0] = ts_entry; t[1] = 0; t[2] = 0; t[3] = wall_clock64();
+    t[0] = ts_entry; t[1] = c.ts[1]; t[2] = c.ts[2]; t[3] = wall_clock64();
   }
 #endif
 }

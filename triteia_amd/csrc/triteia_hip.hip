@@ -73,18 +73,19 @@ void launch_one(const Sparse24Args& a, dim3 grid, hipStream_t st) {
   hipLaunchKernelGGL((sparse24_grouped_kernel<NT, KW, DEPTH>), grid, dim3(64 * KW), 0, st, a);
 }
 
-// `nt`: token tile class; `tsplit`: workgroups along y sharing one group's tokens (legacy / uniform
-// group forms only; plan tiles never exceed one pass).
+// `nt`: token tile class; `tsplit`: workgroups along y sharing one group's tokens (run-table form
+// only: plan tiles never exceed one pass, uniform groups are cut into chunks by the kernel).
 int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   if (tsplit < 1) tsplit = 1;
   if (tsplit > 65535) tsplit = 65535;
-  const long units = (long)a.n_groups * (a.m / 128);
-  if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
-  const dim3 grid((unsigned)units, (unsigned)tsplit);
+  const long cb_pad = (a.m / 128 + 7) / 8 * 8;   // column blocks padded to the 8 XCDs
   const int kw = env_int("TRITEIA_HIP_KW", 4);
   // register budget: two steps in flight for the narrow tiles, one for the 64-token tile
   const int depth = env_int("TRITEIA_HIP_DEPTH", nt == 4 ? 1 : 2);
+  const long units = (long)a.n_groups * cb_pad;
+  if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
+  const dim3 grid((unsigned)units, (unsigned)tsplit);
 #define TRY(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
   TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 2)
   TRY(2, 4, 1) TRY(2, 4, 2) TRY(2, 8, 1)
