@@ -106,13 +106,17 @@ TRITEIA_HIP_API int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, co
 TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n_deltas);
 
 /* Only the routing step of the call above: fills `workspace` (16-byte aligned) with
- *   int32 header[4] = {tiles, routed tokens, deltas in use, tile size}
+ *   int32 header[8] = {narrow tiles, routed tokens, deltas in use, narrow tile size,
+ *                      wide tiles, 0, 0, 0}
  *   int32 tiles[max_tiles][4] = {delta, start, count, 0}: at most `tile size` tokens of one
  *         delta, listed at perm[start .. start+count); a delta's tiles are adjacent
+ *   int32 wide[max_wide][4]   = the same for 64-token tiles; only batches of at least 96
+ *         tokens get any: a delta with c tokens then has c/64 full wide tiles, one more if
+ *         the rest exceeds 32 tokens, and narrow tiles for a smaller rest
  *   int32 perm[prob_n] = token rows grouped by delta, original order kept (stable)
- * with max_tiles = min(prob_n, n_deltas) + prob_n / 16.  The tile size is
- * triteia_hip_plan_tile_tokens(prob_n, n_deltas).  Exposed so that one routing pass can
- * serve every layer of a forward pass and the LoRA path. */
+ * with max_tiles = min(prob_n, n_deltas) + prob_n / 16 and max_wide = prob_n / 33 + 1.  The
+ * narrow tile size is triteia_hip_plan_tile_tokens(prob_n, n_deltas).  Exposed so that one
+ * routing pass can serve every layer of a forward pass and the LoRA path. */
 TRITEIA_HIP_API int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
                            size_t workspace_bytes, int dev, void* stream);
 

@@ -35,6 +35,7 @@ def ops():
 @pytest.mark.parametrize("n,k,m,seed", [
     (1, 128, 256, 1), (3, 512, 256, 2), (16, 512, 256, 3), (17, 512, 256, 4), (64, 512, 384, 5),
     (100, 1024, 256, 6), (5, 192, 128, 7),            # k = 64 (mod 128): the partial last k step
+    (64, 256, 128, 8), (97, 320, 640, 9), (130, 192, 384, 10), (200, 512, 1408, 12),   # wide tiles, ragged ends
     (16, 4096, 4096, 1000),                           # BASELINE config 0
 ])
 def test_matmul_4bit_2_4(ops, n, k, m, seed):
@@ -164,19 +165,30 @@ def test_sbmm_variants(ops, kind, T, N, m, k, sort, seed):
     # -1 rows are exactly zero, routed rows are not
     none = torch.from_numpy(idx < 0).to(DEV)
     assert bool((native[none] == 0).all())
-    # routing is bit-exact: every row equals the single-matrix product of that row alone
+    # routing is exact: every row equals the single-matrix product of that row alone -- bit for
+    # bit when both take the narrow kernel (same K order), to fp32-reassociation accuracy when the
+    # row sits in a 64-token wide tile (one wavefront sums K in order instead of four in parallel)
+    counts = np.bincount(idx[idx >= 0], minlength=N)
     for t in range(0, T, max(1, T // 8)):
         if idx[t] >= 0:
             alone = ops.matmul_4bit_2_4(gq[idx[t]], gx[t:t + 1], gm[idx[t]], gs[idx[t]])
-            assert torch.equal(alone[0], native[t]), f"row {t} differs from its own delta's product"
+            if T < 96 or counts[idx[t]] <= 32:
+                assert torch.equal(alone[0], native[t]), f"row {t} differs from its own delta's product"
+            else:
+                err = (alone[0].float() - native[t].float()).norm() / alone[0].float().norm()
+                assert float(err) < 1e-3, f"row {t}: {float(err):.2e} from its own delta's product"
     forloop = ops.sbmm_4bit_2_4_forloop(gq, gx, gm, gs, gi)
     check_close(forloop, ref, what="sbmm forloop")
-    assert torch.equal(forloop, native)
+    if T < 96:
+        assert torch.equal(forloop, native)
     if sort:
         multi = ops.sbmm_4bit_2_4_multilaunch(gq, gx, gm, gs, gi)
         runs = ops.sbmm_4bit_2_4_runs(gq, gx, gm, gs, gi)
         torch.cuda.synchronize()
-        assert torch.equal(multi, native) and torch.equal(runs, native)
+        check_close(multi, ref, what="sbmm multilaunch")
+        check_close(runs, ref, what="sbmm runs")
+        if T < 96:
+            assert torch.equal(multi, native) and torch.equal(runs, native)
 
 
 def test_sbmm_with_base_weight_accumulates_in_place(ops):
@@ -207,21 +219,33 @@ def test_route_plan_is_a_stable_grouping():
         d = idx - off
         valid = (d >= 0) & (d < N)
         tile = _ffi.lib().triteia_hip_plan_tile_tokens(T, N)
-        max_tiles = min(T, N) + T // 16
-        n_tiles, n_routed, n_used, tile_dev = plan[0], plan[1], plan[2], plan[3]
-        tiles = plan[4:4 + 4 * max_tiles].reshape(max_tiles, 4)[:n_tiles]
-        perm = plan[4 + 4 * max_tiles:4 + 4 * max_tiles + T]
+        max_tiles, max_wide = min(T, N) + T // 16, T // 33 + 1
+        n_tiles, n_routed, n_used, tile_dev, n_wide = plan[0], plan[1], plan[2], plan[3], plan[4]
+        o_tiles, o_wide, o_perm = 8, 8 + 4 * max_tiles, 8 + 4 * max_tiles + 4 * max_wide
+        tiles = plan[o_tiles:o_tiles + 4 * max_tiles].reshape(max_tiles, 4)[:n_tiles]
+        wides = plan[o_wide:o_wide + 4 * max_wide].reshape(max_wide, 4)[:n_wide]
+        perm = plan[o_perm:o_perm + T]
         used = np.unique(d[valid])
         assert tile_dev == tile and n_used == len(used) and n_routed == valid.sum()
-        pos, ti = 0, 0
+        has_wide = T >= 96
+        pos, ti, wi = 0, 0, 0
         for delta in used:
             rows = np.nonzero(d == delta)[0]                # ascending = original order
-            assert np.array_equal(perm[pos:pos + len(rows)], rows)
-            for first in range(0, len(rows), tile):          # the delta's tiles, in order, adjacent
-                assert list(tiles[ti]) == [delta, pos + first, min(tile, len(rows) - first), 0]
+            c = len(rows)
+            assert np.array_equal(perm[pos:pos + c], rows)
+            c_wide = 0
+            if has_wide:
+                c_wide = c // 64 * 64
+                if c - c_wide >= 33:
+                    c_wide = c
+            for first in range(0, c_wide, 64):               # wide tiles first ...
+                assert list(wides[wi]) == [delta, pos + first, min(64, c_wide - first), 0]
+                wi += 1
+            for first in range(c_wide, c, tile):             # ... then the narrow rest
+                assert list(tiles[ti]) == [delta, pos + first, min(tile, c - first), 0]
                 ti += 1
-            pos += len(rows)
-        assert ti == n_tiles
+            pos += c
+        assert ti == n_tiles and wi == n_wide
 
 
 # ------------------------------------------------------------- lora / ldmm

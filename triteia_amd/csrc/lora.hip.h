@@ -94,8 +94,10 @@ struct SgmvArgs {
   // routing plan's tile list {adapter, start, count, 0} + perm
   const int* seg;
   const int4* tiles;
+  const int4* tiles2;         // second tile list (the plan's wide tiles), after the first
   const int* perm;
   const int* n_groups_dev;
+  const int* n_groups2_dev;
   int n_groups;
   int n_adapters;
   float scale;
@@ -108,14 +110,15 @@ struct SgmvGroup {
 
 __device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* out) {
   const int n = a.n_groups_dev ? *a.n_groups_dev : a.n_groups;
-  if (g >= n) return false;
+  const int n2 = a.n_groups2_dev ? *a.n_groups2_dev : 0;
+  if (g >= n + n2) return false;
   int adapter;
   if (a.seg) {
     adapter = g;
     out->start = a.seg[g];
     out->count = a.seg[g + 1] - a.seg[g];
   } else {
-    const int4 d = a.tiles[g];
+    const int4 d = g < n ? a.tiles[g] : a.tiles2[g - n];
     adapter = d.x;
     out->start = d.y;
     out->count = d.z;

@@ -7,11 +7,15 @@
 // indices in any order with -1 (no delta) anywhere.
 //
 // Output (all int32, in the caller's workspace):
-//   header[0] = number of tiles, header[1] = number of routed tokens,
-//   header[2] = number of deltas that have at least one token, header[3] = tile size
+//   header[0] = number of narrow tiles, header[1] = number of routed tokens,
+//   header[2] = number of deltas that have at least one token, header[3] = narrow tile size,
+//   header[4] = number of wide tiles, header[5..7] = 0
 //   tiles[..] = {delta, start, count, 0}: `count` <= tile size tokens of one delta,
 //               listed at perm[start .. start+count); ascending delta id, a delta's
 //               tiles are adjacent
+//   wide[..]  = same, for 64-token tiles (only when built with wide = 1): a delta with c
+//               tokens gets c/64 full wide tiles, one more if the rest exceeds 32 tokens,
+//               and narrow tiles for a smaller rest
 //   perm[routed] = token rows, grouped by delta, original order kept inside a
 //               delta (stable)
 #pragma once
@@ -20,14 +24,16 @@
 
 namespace triteia_hip {
 
-constexpr int kPlanHeaderInts = 4;
+constexpr int kPlanHeaderInts = 8;
+constexpr int kPlanWideTile = 64;      // tokens per wide tile
+constexpr int kPlanWideMinRest = 33;   // a rest of at least this many tokens still forms a wide tile
 constexpr int kPlanMaxDeltas = 8192;  // per-delta cursors live in LDS
 constexpr int kPlanThreads = 256;
 constexpr int kPlanMinTile = 16;      // smallest tile size a plan can be built for
 
 struct PlanLayout {
-  int header, tiles, perm, total;  // offsets in ints
-  int max_tiles;
+  int header, tiles, wide, perm, total;  // offsets in ints
+  int max_tiles, max_wide;
 };
 
 // The layout depends only on (tokens, deltas), not on the tile size the plan is built
@@ -36,9 +42,11 @@ __host__ __device__ inline PlanLayout plan_layout(int n_tokens, int n_deltas) {
   const int g = n_deltas < n_tokens ? n_deltas : n_tokens;
   PlanLayout l;
   l.max_tiles = g + n_tokens / kPlanMinTile;
+  l.max_wide = n_tokens / kPlanWideMinRest + 1;
   l.header = 0;
   l.tiles = kPlanHeaderInts;
-  l.perm = l.tiles + 4 * l.max_tiles;
+  l.wide = l.tiles + 4 * l.max_tiles;
+  l.perm = l.wide + 4 * l.max_wide;
   l.total = l.perm + n_tokens;
   return l;
 }
@@ -61,7 +69,7 @@ __device__ __forceinline__ int wave_excl_scan(int v, int lane, int* total) {
 
 // One workgroup.  indices[t] - index_offset outside [0, n_deltas) means "no delta".
 __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __restrict__ indices, int n_tokens,
-                                                                 int n_deltas, int index_offset, int tile,
+                                                                 int n_deltas, int index_offset, int tile, int wide,
                                                                  int* __restrict__ ws) {
   __shared__ int s_cursor[kPlanMaxDeltas];
   const PlanLayout L = plan_layout(n_tokens, n_deltas);
@@ -79,22 +87,37 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
   if (tid < 64) {
     // exclusive scans over the deltas, 64 per iteration: token counts -> first slot in perm,
     // tile counts -> first tile
-    int running = 0, tiles = 0, groups = 0;
+    int running = 0, tiles = 0, wides = 0, groups = 0;
     int4* tile_out = reinterpret_cast<int4*>(ws + L.tiles);
+    int4* wide_out = reinterpret_cast<int4*>(ws + L.wide);
     for (int base = 0; base < n_deltas; base += 64) {
       const int d = base + lane;
       const int c = d < n_deltas ? s_cursor[d] : 0;
-      int chunk_tokens, chunk_tiles;
+      int chunk_tokens, chunk_tiles, chunk_wides;
       const int offs = running + wave_excl_scan(c, lane, &chunk_tokens);
-      const int nt = (c + tile - 1) / tile;
+      // split this delta's tokens: wide tiles first, the rest in narrow tiles
+      int nw = 0, c_wide = 0;
+      if (wide) {
+        nw = c / kPlanWideTile;
+        c_wide = nw * kPlanWideTile;
+        if (c - c_wide >= kPlanWideMinRest) { nw++; c_wide = c; }
+      }
+      const int c_rest = c - c_wide;
+      const int nt = (c_rest + tile - 1) / tile;
+      const int wpos = wides + wave_excl_scan(nw, lane, &chunk_wides);
       const int tpos = tiles + wave_excl_scan(nt, lane, &chunk_tiles);
+      for (int i = 0; i < nw; i++) {
+        const int first = i * kPlanWideTile;
+        wide_out[wpos + i] = make_int4(d, offs + first, min(kPlanWideTile, c_wide - first), 0);
+      }
       for (int i = 0; i < nt; i++) {
         const int first = i * tile;
-        tile_out[tpos + i] = make_int4(d, offs + first, min(tile, c - first), 0);
+        tile_out[tpos + i] = make_int4(d, offs + c_wide + first, min(tile, c_rest - first), 0);
       }
       if (d < n_deltas) s_cursor[d] = offs;
       running += chunk_tokens;
       tiles += chunk_tiles;
+      wides += chunk_wides;
       groups += __popcll(__ballot(c > 0));
     }
     if (lane == 0) {
@@ -102,6 +125,10 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
       ws[L.header + 1] = running;
       ws[L.header + 2] = groups;
       ws[L.header + 3] = tile;
+      ws[L.header + 4] = wides;
+      ws[L.header + 5] = 0;
+      ws[L.header + 6] = 0;
+      ws[L.header + 7] = 0;
     }
     // stable placement: 64 tokens at a time, tokens with equal delta ranked by lane order
     for (int base = 0; base < n_tokens; base += 64) {

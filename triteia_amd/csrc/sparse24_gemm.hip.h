@@ -65,7 +65,8 @@ struct Sparse24Args {
   // groups, one of three forms:
   //   tiles   : packed {delta, start, count, 0} per group (the routing plan's tile list)
   //   g_*     : three separate arrays (the reference's run table)
-  //   neither : group j = delta j*delta_step with rows [j*uniform_count, (j+1)*uniform_count)
+  //   neither : group j = delta j*delta_step with uniform_count rows from
+  //             j*uniform_stride + uniform_first
   const int4* tiles;
   const int* g_delta;
   const int* g_start;
@@ -74,6 +75,8 @@ struct Sparse24Args {
   const int* n_groups_dev;  // device-side group count (nullptr: n_groups)
   int n_groups;             // upper bound on the number of groups
   int uniform_count;
+  int uniform_stride;
+  int uniform_first;
   int delta_step;
   int n_deltas;             // deltas with index outside [0, n_deltas) are skipped
   int accumulate;           // 0: out = result, 1: out += result
@@ -347,7 +350,7 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
     count = p.g_count[grp];
   } else {
     delta = grp * p.delta_step;
-    start = grp * p.uniform_count;
+    start = grp * p.uniform_stride + p.uniform_first;
     count = p.uniform_count;
   }
   const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;

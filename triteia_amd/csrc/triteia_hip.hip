@@ -12,6 +12,7 @@
 #include "lora.hip.h"
 #include "route_plan.hip.h"
 #include "sparse24_gemm.hip.h"
+#include "sparse24_wide.hip.h"
 
 namespace {
 
@@ -113,12 +114,62 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.g_delta = a.g_start = a.g_count = a.perm = a.n_groups_dev = nullptr;
   a.n_groups = 0;
   a.uniform_count = 0;
+  a.uniform_stride = 0;
+  a.uniform_first = 0;
   a.delta_step = 0;
   a.accumulate = 0;
   a.xcd_swizzle = env_int("TRITEIA_HIP_XCD_SWIZZLE", 1);
 #ifdef TRITEIA_HIP_TIMELINE
   a.timeline = reinterpret_cast<long long*>(strtoull(getenv("TRITEIA_HIP_TIMELINE_PTR") ? getenv("TRITEIA_HIP_TIMELINE_PTR") : "0", nullptr, 0));
 #endif
+}
+
+
+// Wide (64-token x 512-column) tiles: groups from a plan's wide list or uniform groups.
+int launch_wide(const Sparse24Args& a, hipStream_t st) {
+  if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
+  const long cgs = (a.m / 128 + 3) / 4;
+  const long cg_pad = (cgs + 7) / 8 * 8;
+  const long chunks = a.tiles ? 1 : (a.uniform_count + kWideTokens - 1) / kWideTokens;
+  const long units = (long)a.n_groups * chunks * cg_pad;
+  if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
+  Sparse24Args b = a;
+  if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
+  if (env_int("TRITEIA_HIP_WIDE_DEPTH", 2) == 1)
+    hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3((unsigned)units), dim3(256), 0, st, b);
+  else
+    hipLaunchKernelGGL((sparse24_wide_kernel<2>), dim3((unsigned)units), dim3(256), 0, st, b);
+  return check_launch("sparse24_wide_kernel");
+}
+
+// tokens per group from which the wide kernel takes over (0 = never)
+int wide_threshold() { return env_int("TRITEIA_HIP_WIDE_MIN", 64); }
+
+// `tokens` rows per group, `stride` rows between groups: full 64-token chunks (and a rest above
+// 32 tokens) go to the wide kernel, what is left to the narrow one.
+int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n_groups, hipStream_t st) {
+  a.n_groups = n_groups;
+  a.uniform_stride = stride;
+  a.delta_step = delta_step;
+  int wide_tokens = 0;
+  const int wmin = wide_threshold();
+  if (wmin > 0 && tokens >= wmin) {
+    wide_tokens = tokens / kWideTokens * kWideTokens;
+    if (tokens - wide_tokens >= kPlanWideMinRest) wide_tokens = tokens;
+  }
+  if (wide_tokens > 0) {
+    a.uniform_first = 0;
+    a.uniform_count = wide_tokens;
+    if (int e = launch_wide(a, st)) return e;
+  }
+  const int rest = tokens - wide_tokens;
+  if (rest > 0) {
+    a.uniform_first = wide_tokens;
+    a.uniform_count = rest;
+    const int nt = pick_nt(rest, 1);
+    return launch_sparse24(a, nt, (rest + 16 * nt - 1) / (16 * nt), st);
+  }
+  return TRITEIA_HIP_OK;
 }
 
 }  // namespace
@@ -140,10 +191,7 @@ int triteia_hip_mul_2_4(const void* A, const void* B, const void* meta, void* C,
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   Sparse24Args a;
   fill_weights(a, A, B, meta, C, s, prob_m, prob_k, 1);
-  a.n_groups = 1;
-  a.uniform_count = prob_n;
-  const int nt = pick_nt(prob_n, 1);
-  return launch_sparse24(a, nt, (prob_n + 16 * nt - 1) / (16 * nt), static_cast<hipStream_t>(stream));
+  return launch_uniform(a, prob_n, prob_n, 0, 1, static_cast<hipStream_t>(stream));
 }
 
 int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
@@ -156,11 +204,7 @@ int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, v
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   Sparse24Args a;
   fill_weights(a, A, B, meta, C, s, prob_m, prob_k, batch);
-  a.n_groups = batch;
-  a.uniform_count = tokens;
-  a.delta_step = 1;
-  const int nt = pick_nt(tokens, 1);
-  return launch_sparse24(a, nt, (tokens + 16 * nt - 1) / (16 * nt), static_cast<hipStream_t>(stream));
+  return launch_uniform(a, tokens, tokens, 1, batch, static_cast<hipStream_t>(stream));
 }
 
 int triteia_hip_bmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m, int prob_n,
@@ -205,6 +249,12 @@ int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas) {
   return 16 * pick_nt(prob_n, prob_n < n_deltas ? prob_n : n_deltas);
 }
 
+// a plan carries wide (64-token) tiles only when the batch is large enough to have any
+static int plan_has_wide(int prob_n) {
+  const int wmin = wide_threshold();
+  return wmin > 0 && prob_n >= wmin + 32;
+}
+
 int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
                            size_t workspace_bytes, int dev, void* stream) {
   if (prob_n < 0 || n_deltas < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "route_plan: tokens=%d deltas=%d", prob_n, n_deltas);
@@ -220,7 +270,7 @@ int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_de
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   hipLaunchKernelGGL(route_plan_kernel, dim3(1), dim3(kPlanThreads), 0, static_cast<hipStream_t>(stream),
                      static_cast<const int*>(token_indices), prob_n, n_deltas, index_offset,
-                     triteia_hip_plan_tile_tokens(prob_n, n_deltas), static_cast<int*>(workspace));
+                     triteia_hip_plan_tile_tokens(prob_n, n_deltas), plan_has_wide(prob_n), static_cast<int*>(workspace));
   return check_launch("route_plan_kernel");
 }
 
@@ -244,7 +294,14 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
   a.n_groups_dev = ws + L.header;
   a.n_groups = plan_max_tiles(prob_n, n_deltas, tile);
   a.accumulate = accumulate;
-  return launch_sparse24(a, tile / 16, 1, static_cast<hipStream_t>(stream));
+  if (int e = launch_sparse24(a, tile / 16, 1, static_cast<hipStream_t>(stream))) return e;
+  if (plan_has_wide(prob_n)) {
+    a.tiles = reinterpret_cast<const int4*>(ws + L.wide);
+    a.n_groups_dev = ws + L.header + 4;
+    a.n_groups = L.max_wide;
+    return launch_wide(a, static_cast<hipStream_t>(stream));
+  }
+  return TRITEIA_HIP_OK;
 }
 
 int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, void* C, const void* s,
@@ -361,6 +418,11 @@ int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride
   a.perm = ws + L.perm;
   a.n_groups_dev = ws + L.header;
   a.n_groups = plan_max_tiles(prob_n, n_adapters, triteia_hip_plan_tile_tokens(prob_n, n_adapters));
+  if (plan_has_wide(prob_n)) {
+    a.tiles2 = reinterpret_cast<const int4*>(ws + L.wide);
+    a.n_groups2_dev = ws + L.header + 4;
+    a.n_groups += L.max_wide;
+  }
   a.n_adapters = n_adapters;
   a.scale = scale;
   return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream));
