@@ -110,8 +110,8 @@ TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n
  *                      wide tiles, 0, 0, 0}
  *   int32 tiles[max_tiles][4] = {delta, start, count, 0}: at most `tile size` tokens of one
  *         delta, listed at perm[start .. start+count); a delta's tiles are adjacent
- *   int32 wide[max_wide][4]   = the same for 64-token tiles; only batches of at least 96
- *         tokens get any: a delta with c tokens then has c/64 full wide tiles, one more if
+ *   int32 wide[max_wide][4]   = the same for 64-token tiles; only batches of at least 4096
+ *         tokens (environment TRITEIA_HIP_WIDE_MIN_BATCH) get any: a delta with c tokens then has c/64 full wide tiles, one more if
  *         the rest exceeds 32 tokens, and narrow tiles for a smaller rest
  *   int32 perm[prob_n] = token rows grouped by delta, original order kept (stable)
  * with max_tiles = min(prob_n, n_deltas) + prob_n / 16 and max_wide = prob_n / 33 + 1.  The

@@ -19,6 +19,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+WIDE_MIN_BATCH = 512          # the tests lower the batch size from which plans carry wide tiles
+
+
+@pytest.fixture(autouse=True)
+def _wide_tiles_from_512_tokens(monkeypatch):
+    monkeypatch.setenv("TRITEIA_HIP_WIDE_MIN_BATCH", str(WIDE_MIN_BATCH))
+
+
 def say(msg):
     print(f"[case] {msg}", flush=True)
     sys.stdout.flush()
@@ -151,6 +159,8 @@ def _indices(kind, T, N, seed, sort):
     ("none", 9, 3, 256, 128, True, 35),              # all -1
     ("single", 40, 3, 256, 256, True, 36),           # one run
     ("uniform", 64, 16, 4096, 4096, False, 1002),    # BASELINE config 2
+    ("zipf", 600, 6, 512, 256, False, 37),           # plan with wide (64-token) tiles
+    ("zipf", 700, 5, 640, 192, False, 38),           # the same with a partial last K step
 ])
 def test_sbmm_variants(ops, kind, T, N, m, k, sort, seed):
     say(f"sbmm {kind} T={T} N={N} m={m} k={k} sorted={sort} seed={seed}")
@@ -172,14 +182,14 @@ def test_sbmm_variants(ops, kind, T, N, m, k, sort, seed):
     for t in range(0, T, max(1, T // 8)):
         if idx[t] >= 0:
             alone = ops.matmul_4bit_2_4(gq[idx[t]], gx[t:t + 1], gm[idx[t]], gs[idx[t]])
-            if T < 96 or counts[idx[t]] <= 32:
+            if T < 512 or counts[idx[t]] <= 32:
                 assert torch.equal(alone[0], native[t]), f"row {t} differs from its own delta's product"
             else:
                 err = (alone[0].float() - native[t].float()).norm() / alone[0].float().norm()
                 assert float(err) < 1e-3, f"row {t}: {float(err):.2e} from its own delta's product"
     forloop = ops.sbmm_4bit_2_4_forloop(gq, gx, gm, gs, gi)
     check_close(forloop, ref, what="sbmm forloop")
-    if T < 96:
+    if T < 512:
         assert torch.equal(forloop, native)
     if sort:
         multi = ops.sbmm_4bit_2_4_multilaunch(gq, gx, gm, gs, gi)
@@ -187,7 +197,7 @@ def test_sbmm_variants(ops, kind, T, N, m, k, sort, seed):
         torch.cuda.synchronize()
         check_close(multi, ref, what="sbmm multilaunch")
         check_close(runs, ref, what="sbmm runs")
-        if T < 96:
+        if T < 512:
             assert torch.equal(multi, native) and torch.equal(runs, native)
 
 
@@ -213,7 +223,7 @@ def test_route_plan_is_a_stable_grouping():
     from triteia_amd.python.capi import _ffi, route_plan
     say("route plan")
     rng = np.random.default_rng(51)
-    for T, N, off in [(1, 1, 0), (64, 16, 0), (200, 7, 0), (1000, 300, 0), (130, 5, 3), (70, 100, 0), (700, 3, 0)]:
+    for T, N, off in [(1, 1, 0), (64, 16, 0), (200, 7, 0), (1000, 300, 0), (130, 5, 3), (70, 100, 0), (700, 3, 0), (520, 40, 0)]:
         idx = rng.integers(-1, N + off, size=T).astype(np.int32)
         plan = route_plan(torch.from_numpy(idx).to(DEV), N, index_offset=off).cpu().numpy()
         d = idx - off
@@ -227,7 +237,7 @@ def test_route_plan_is_a_stable_grouping():
         perm = plan[o_perm:o_perm + T]
         used = np.unique(d[valid])
         assert tile_dev == tile and n_used == len(used) and n_routed == valid.sum()
-        has_wide = T >= 96
+        has_wide = T >= 512
         pos, ti, wi = 0, 0, 0
         for delta in used:
             rows = np.nonzero(d == delta)[0]                # ascending = original order

@@ -7,25 +7,28 @@
 //   * a workgroup owns a 64-token x 512-column tile: its 4 wavefronts take 4
 //     adjacent 128-column blocks and each runs the whole K range (no K split, no
 //     cross-wave reduction; every dequantised weight fragment feeds 4 MFMAs);
-//   * the 64 x 128 activation tile of each K step is fetched from global memory
-//     once per workgroup into LDS (double buffered) and read by all 4 wavefronts,
-//     instead of once per wavefront: one barrier per K step;
+//   * the 64 x 128 activation tile of each K step is fetched once per workgroup,
+//     straight from global memory into LDS (global_load_lds_dwordx4, no registers in
+//     between), three steps ahead of its use in a 4-stage ring, and read by all 4
+//     wavefronts: one barrier per K step;
 //   * outputs go straight from the accumulators to memory (each lane holds 32
 //     consecutive features of one token).
-// LDS rows are padded to 272 B so that the 16 token rows read by one
-// ds_read_b128 fall into distinct banks.
+// An LDS row is the 256 B of one token; the 16-byte chunk c of row n is stored at chunk
+// position c ^ (n % 16), so that the 16 token rows read by one ds_read_b128 fall into
+// distinct banks while every direct-to-LDS load still writes 1 KB of consecutive LDS.
+// Needs k % 128 == 0 (a direct load cannot zero-fill a partial K step).
 #pragma once
 #include "sparse24_gemm.hip.h"
 
 namespace triteia_hip {
 
 constexpr int kWideTokens = 64;
-constexpr int kWideRowHalfs = 136;   // 128 k + 8 halfs of padding
+constexpr int kWideStages = 4;        // activation tiles in flight (LDS ring)
 
 template <int DEPTH>
-__global__ __launch_bounds__(256) void sparse24_wide_kernel(const Sparse24Args p) {
+__global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Args p) {
   constexpr int NT = kWideTokens / 16;
-  __shared__ _Float16 xs[2][kWideTokens][kWideRowHalfs];
+  __shared__ __attribute__((aligned(1024))) _Float16 xs[kWideStages][kWideTokens][128];
   __shared__ int s_rows[kWideTokens];
 
   const int tid = threadIdx.x;
@@ -81,25 +84,23 @@ __global__ __launch_bounds__(256) void sparse24_wide_kernel(const Sparse24Args p
   }
   __syncthreads();
 
-  // cooperative activation fetch: thread t moves 16-byte chunk (t % 16) of rows t/16 + 16 i
-  const int xc = tid & 15;
+  // cooperative activation fetch.  One direct-to-LDS instruction of a wavefront writes 64
+  // consecutive 16-byte chunks = 4 token rows; instruction ii of wave w covers rows
+  // 16 ii + 4 w + lane/16.  Lane l fills chunk position l % 16 of its row, which holds the
+  // row's chunk (l % 16) ^ (row % 16).
   const _Float16* xsrc[4];
 #pragma unroll
-  for (int ii = 0; ii < 4; ii++) xsrc[ii] = p.x + (long)s_rows[(tid >> 4) + 16 * ii] * p.x_stride + xc * 8;
-  uint4_t xg[4];
-  auto load_xg = [&](int st) {
-    // the last step may be half empty (k % 128 == 64): chunks past K are zeroed at the store
-    const int koff = min(st * 128 + xc * 8, p.k - 8) - xc * 8;
+  for (int ii = 0; ii < 4; ii++) {
+    const int row = 16 * ii + 4 * wave + (lane >> 4);
+    const int chunk = (lane & 15) ^ (row & 15);
+    xsrc[ii] = p.x + (long)s_rows[row] * p.x_stride + chunk * 8;
+  }
+  auto issue_x = [&](int st) {
+    const int stc = min(st, n_steps - 1);   // past the end: refetch the last tile (never read)
+    const int stage = st & (kWideStages - 1);
 #pragma unroll
-    for (int ii = 0; ii < 4; ii++) xg[ii] = *reinterpret_cast<const uint4_t*>(xsrc[ii] + koff);
-  };
-  auto store_xg = [&](int stage, int st) {
-    const bool in_k = st * 128 + xc * 8 < p.k;
-#pragma unroll
-    for (int ii = 0; ii < 4; ii++) {
-      const uint4_t v = in_k ? xg[ii] : uint4_t{0u, 0u, 0u, 0u};
-      *reinterpret_cast<uint4_t*>(&xs[stage][(tid >> 4) + 16 * ii][xc * 8]) = v;
-    }
+    for (int ii = 0; ii < 4; ii++)
+      __builtin_amdgcn_global_load_lds(xsrc[ii] + stc * 128, &xs[stage][16 * ii + 4 * wave][0], 16, 0, 0);
   };
 
   struct WFrag {
@@ -126,66 +127,82 @@ __global__ __launch_bounds__(256) void sparse24_wide_kernel(const Sparse24Args p
   // B operand of lane (n = r, qb = q): k offsets 8*(q%2) + {0..7} of packed rows q/2 and 2 + q/2
   // of the step, i.e. halfs [32*(q/2) + 8*(q%2) + 16u, +8) and the same + 64
   const int xb_off = 32 * (q >> 1) + 8 * (q & 1);
+  // reads the B fragment (16 halfs) of 16-token tile nt, k-half u from the LDS stage
+  auto read_b = [&](int stage, int nt, int u) {
+    // chunks c and c + 8 of token row nt*16 + r, at their swizzled positions
+    const int c = (xb_off >> 3) + 2 * u;
+    const _Float16* row = &xs[stage][nt * 16 + r][0];
+    typedef uint32_t uint8_t_v __attribute__((ext_vector_type(8)));
+    const uint4_t lo = *reinterpret_cast<const uint4_t*>(row + ((c ^ r) << 3));
+    const uint4_t hi = *reinterpret_cast<const uint4_t*>(row + (((c + 8) ^ r) << 3));
+    const uint8_t_v bb = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(half16_t, bb);
+  };
   auto compute_step = [&](const WFrag& f, int stage) {
+    // Per k-half u and per half of the 8 columns: dequantise 4 weight fragments, then run them
+    // against the four 16-token B fragments.  B fragments are read one ahead of the MFMAs that
+    // use them, so that the LDS latency hides behind 4 MFMAs instead of stalling in front of them.
+    half16_t b_nxt = read_b(stage, 0, 0);
 #pragma unroll
     for (int u = 0; u < 2; u++) {
-      half8_t A[8];
-      int idx[8];
 #pragma unroll
-      for (int cc = 0; cc < 8; cc++) {
-        const int w = cc & 3;
-        const int b2 = cc >> 2;
-        uint4_t av;
+      for (int b2 = 0; b2 < 2; b2++) {
+        half8_t A[4];
 #pragma unroll
-        for (int a = 0; a < 4; a++) {
-          uint32_t word = f.wq[a][w];
-          if (b2) word >>= 8;
-          av[a] = u ? dequant_odd(word) : dequant_even(word);
+        for (int w = 0; w < 4; w++) {
+          uint4_t av;
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            uint32_t word = f.wq[a][w];
+            if (b2) word >>= 8;
+            av[a] = u ? dequant_odd(word) : dequant_even(word);
+          }
+          A[w] = __builtin_bit_cast(half8_t, av);
         }
-        A[cc] = __builtin_bit_cast(half8_t, av);
-        idx[cc] = (int)f.mt[(cc >> 1) & 1][(cc & 1) * 2 + u];
-      }
 #pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        const _Float16* row = &xs[stage][nt * 16 + r][xb_off + 16 * u];
-        typedef uint32_t uint8_t_v __attribute__((ext_vector_type(8)));
-        const uint4_t lo = *reinterpret_cast<const uint4_t*>(row);
-        const uint4_t hi = *reinterpret_cast<const uint4_t*>(row + 64);
-        const uint8_t_v bb = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        const half16_t b = __builtin_bit_cast(half16_t, bb);
+        for (int nt = 0; nt < NT; nt++) {
+          const half16_t b = b_nxt;
+          if (nt + 1 < NT) b_nxt = read_b(stage, nt + 1, u);
+          else if (b2 == 0) b_nxt = read_b(stage, 0, u);
+          else if (u == 0) b_nxt = read_b(stage, 0, 1);
 #pragma unroll
-        for (int cc = 0; cc < 8; cc++) {
-          if (cc >> 2)
-            acc[cc][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A[cc], b, acc[cc][nt], idx[cc], 0, 1);
-          else
-            acc[cc][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A[cc], b, acc[cc][nt], idx[cc], 0, 0);
+          for (int w = 0; w < 4; w++) {
+            const int cc = 4 * b2 + w;
+            const int idx = (int)f.mt[(cc >> 1) & 1][(cc & 1) * 2 + u];
+            if (b2)
+              acc[cc][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A[w], b, acc[cc][nt], idx, 0, 1);
+            else
+              acc[cc][nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A[w], b, acc[cc][nt], idx, 0, 0);
+          }
         }
       }
     }
   };
 
-  // pipeline: weights DEPTH steps ahead in registers, activations one step ahead through LDS
+  // pipeline: weights DEPTH steps ahead in registers; activation tiles 3 steps ahead in the
+  // LDS ring.  At the top of step st this wave waits until its own direct loads of tile st
+  // have landed (everything it issued since then is allowed to stay in flight: 4 loads for each
+  // of tiles st+1 and st+2 at least), then the barrier makes all four waves' parts visible
+  // and also says that tile st-1 has been read by everyone, so its stage can be refilled.
   WFrag ring[DEPTH];
 #pragma unroll
   for (int j = 0; j < DEPTH; j++) load_w(ring[j], j);
-  load_xg(0);
-  store_xg(0, 0);
-  lds_barrier();
-  constexpr int TURN = DEPTH % 2 == 0 ? DEPTH : 2 * DEPTH;   // whole ring turns and LDS stage pairs
+  issue_x(0);
+  issue_x(1);
+  issue_x(2);
+  constexpr int TURN = DEPTH > 4 ? DEPTH : 4;   // whole ring turns of both rings (DEPTH divides 4)
   for (int s0 = 0; s0 < n_steps; s0 += TURN) {
 #pragma unroll
     for (int j = 0; j < TURN; j++) {
       const int st = s0 + j;
-      // the same loads and stores every iteration (the step after the last one re-reads the
-      // last tile into the stage nobody reads), so that load-counter waits stay exact
-      const int nxt = min(st + 1, n_steps - 1);
-      load_xg(nxt);
-      if (st < n_steps && active) compute_step(ring[j % DEPTH], j & 1);
-      load_w(ring[j % DEPTH], st + DEPTH);
-      store_xg((j + 1) & 1, nxt);
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 8);   // vmcnt(8), nothing else
       lds_barrier();
+      issue_x(st + 3);
+      if (st < n_steps && active) compute_step(ring[j % DEPTH], j & (kWideStages - 1));
+      load_w(ring[j % DEPTH], st + DEPTH);
     }
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): no direct load may outlive the block's LDS
 
   if (!active) return;
   // epilogue: lane (n = r, qq = q) holds features 32q + 8j + c of token n for every 16-token tile

@@ -135,15 +135,17 @@ int launch_wide(const Sparse24Args& a, hipStream_t st) {
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   Sparse24Args b = a;
   if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
-  if (env_int("TRITEIA_HIP_WIDE_DEPTH", 2) == 1)
+  if (env_int("TRITEIA_HIP_WIDE_DEPTH", 1) == 1)
     hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3((unsigned)units), dim3(256), 0, st, b);
   else
     hipLaunchKernelGGL((sparse24_wide_kernel<2>), dim3((unsigned)units), dim3(256), 0, st, b);
   return check_launch("sparse24_wide_kernel");
 }
 
-// tokens per group from which the wide kernel takes over (0 = never)
-int wide_threshold() { return env_int("TRITEIA_HIP_WIDE_MIN", 64); }
+// The wide kernel pays off when there are enough 64-token x 512-column tiles to occupy the
+// GPU; below that the narrow kernel's smaller units win.  TRITEIA_HIP_WIDE=0 disables it.
+bool wide_enabled() { return env_int("TRITEIA_HIP_WIDE", 1) != 0; }
+constexpr long kWideMinUnits = 128;
 
 // `tokens` rows per group, `stride` rows between groups: full 64-token chunks (and a rest above
 // 32 tokens) go to the wide kernel, what is left to the narrow one.
@@ -152,8 +154,8 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   a.uniform_stride = stride;
   a.delta_step = delta_step;
   int wide_tokens = 0;
-  const int wmin = wide_threshold();
-  if (wmin > 0 && tokens >= wmin) {
+  const long cgs = (a.m / 128 + 3) / 4;
+  if (wide_enabled() && a.k % 128 == 0 && (long)n_groups * (tokens / kWideTokens) * cgs >= kWideMinUnits) {
     wide_tokens = tokens / kWideTokens * kWideTokens;
     if (tokens - wide_tokens >= kPlanWideMinRest) wide_tokens = tokens;
   }
@@ -249,10 +251,12 @@ int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas) {
   return 16 * pick_nt(prob_n, prob_n < n_deltas ? prob_n : n_deltas);
 }
 
-// a plan carries wide (64-token) tiles only when the batch is large enough to have any
+// A plan carries wide (64-token) tiles only for batches large enough that whole deltas become
+// bound by the matrix cores (the plan is independent of the layer shape, so the rule only looks
+// at the batch).  Below that, re-reading a hot delta's weights from cache in 32-token tiles is
+// cheaper than a second, poorly filled launch.
 static int plan_has_wide(int prob_n) {
-  const int wmin = wide_threshold();
-  return wmin > 0 && prob_n >= wmin + 32;
+  return wide_enabled() && prob_n >= env_int("TRITEIA_HIP_WIDE_MIN_BATCH", 4096);
 }
 
 int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
@@ -299,7 +303,9 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     a.tiles = reinterpret_cast<const int4*>(ws + L.wide);
     a.n_groups_dev = ws + L.header + 4;
     a.n_groups = L.max_wide;
-    return launch_wide(a, static_cast<hipStream_t>(stream));
+    if (prob_k % 128 == 0) return launch_wide(a, static_cast<hipStream_t>(stream));
+    // a partial last K step needs the narrow kernel: it walks the 64-token tiles in 16*nt-token passes
+    return launch_sparse24(a, tile / 16, (kWideTokens + tile - 1) / tile, static_cast<hipStream_t>(stream));
   }
   return TRITEIA_HIP_OK;
 }
