@@ -65,9 +65,15 @@ struct Sparse24Args {
   // groups, one of three forms:
   //   tiles   : packed {delta, start, count, 0} per group (the routing plan's tile list)
   //   g_*     : three separate arrays (the reference's run table)
-  //   neither : group j = delta j*delta_step with uniform_count rows from
+  //   none    : group j = delta j*delta_step with uniform_count rows from
   //             j*uniform_stride + uniform_first
+  //   raw_indices : (takes precedence) the batch's per-token delta indices, at most 64 tokens
+  //             and 64 deltas: every workgroup derives its group itself ("fused routing"),
+  //             group j = the j-th delta in use, in ascending order
   const int4* tiles;
+  const int* raw_indices;
+  int raw_count;
+  int raw_offset;
   const int* g_delta;
   const int* g_start;
   const int* g_count;
@@ -128,6 +134,7 @@ struct TileCtx {
   int k_rows, n_steps;      // packed rows, 128-k steps
   int cb;                   // column block
   int tid, wave, lane, r, q;
+  int raw_list;             // fused routing: lane s holds the token row of slot s of the group
 #ifdef TRITEIA_HIP_TIMELINE
   long long ts[4];          // debug builds: entry, operands requested, K loop done, end
 #endif
@@ -161,7 +168,8 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 #pragma unroll
   for (int nt = 0; nt < NTT; nt++) {
     const int slot = min(nt * 16 + r, cnt - 1);   // slots past the end re-read the last row
-    rows[nt] = p.perm ? p.perm[first + slot] : first + slot;
+    if (p.raw_indices) rows[nt] = __shfl(c.raw_list, first + slot, 64);
+    else rows[nt] = p.perm ? p.perm[first + slot] : first + slot;
   }
   StepFrag<NTT> ring[DEPTH];
 #pragma unroll
@@ -339,7 +347,37 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
   // group descriptor and live group count are fetched side by side (no dependent chain);
   // grp < p.n_groups (the host's upper bound) keeps the descriptor reads in bounds
   int delta, start, count;
-  if (p.tiles) {
+  int raw_list = 0;
+  if (p.raw_indices) {
+    // Fused routing for small batches: every wavefront looks at all (<= 64) indices, one per
+    // lane, and works out the grp-th delta in use and the rows routed to it -- a few dozen
+    // instructions instead of a separate routing launch and a dependent descriptor read.
+    const int lane_ = threadIdx.x & 63;
+    int d = -1;
+    if (lane_ < p.raw_count) {
+      d = p.raw_indices[lane_] - p.raw_offset;
+      if (d < 0 || d >= p.n_deltas) d = -1;
+    }
+    unsigned long long used = d >= 0 ? (1ull << d) : 0ull;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const unsigned lo = __shfl_xor((unsigned)used, off, 64);
+      const unsigned hi = __shfl_xor((unsigned)(used >> 32), off, 64);
+      used |= ((unsigned long long)hi << 32) | lo;
+    }
+    if (grp >= __popcll(used)) return;
+    const unsigned long long below = (1ull << lane_) - 1ull;
+    const bool is_grp = ((used >> lane_) & 1ull) && __popcll(used & below) == grp;
+    delta = __ffsll((long long)__ballot(is_grp)) - 1;
+    const unsigned long long members = __ballot(d == delta);
+    count = __popcll(members);
+    start = 0;
+    // slot s of the group = the s-th member token: a full permutation sends every member's
+    // token id to the lane of its rank (non-members fill the lanes after the members)
+    const int rank = __popcll(members & below);
+    const int dest = (d == delta) ? rank : count + (lane_ - rank);
+    raw_list = __builtin_amdgcn_ds_permute(dest << 2, lane_);
+  } else if (p.tiles) {
     const int4 d = p.tiles[grp];
     delta = d.x;
     start = d.y;
@@ -364,6 +402,7 @@ __global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse2
   c.r = c.lane & 15;
   c.q = c.lane >> 4;
   c.cb = cb;
+  c.raw_list = raw_list;
   c.k_rows = p.k >> 5;                 // packed rows (32 dense k each)
   c.n_steps = (c.k_rows + 3) >> 2;     // 128 dense k per step
   c.qrow = p.m >> 1;

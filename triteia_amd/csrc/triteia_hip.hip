@@ -111,6 +111,9 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.k = prob_k;
   a.n_deltas = n_deltas;
   a.tiles = nullptr;
+  a.raw_indices = nullptr;
+  a.raw_count = 0;
+  a.raw_offset = 0;
   a.g_delta = a.g_start = a.g_count = a.perm = a.n_groups_dev = nullptr;
   a.n_groups = 0;
   a.uniform_count = 0;
@@ -318,6 +321,20 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: accumulate=%d", accumulate);
   if (prob_m == 0 || prob_n == 0 || prob_k == 0 || n_deltas == 0) return TRITEIA_HIP_OK;
   if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null tensor pointer");
+  if (prob_n <= 64 && n_deltas <= 64 && env_int("TRITEIA_HIP_FUSED_ROUTE", 1)) {
+    // small batch: the multiply kernel routes by itself, no plan, no workspace traffic
+    if (!token_indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null indices");
+    DeviceGuard g(dev);
+    if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+    Sparse24Args a;
+    fill_weights(a, A, B, meta, C, s, prob_m, prob_k, n_deltas);
+    a.raw_indices = static_cast<const int*>(token_indices);
+    a.raw_count = prob_n;
+    a.raw_offset = index_offset;
+    a.n_groups = prob_n < n_deltas ? prob_n : n_deltas;
+    a.accumulate = accumulate;
+    return launch_sparse24(a, pick_nt(prob_n, a.n_groups), 1, static_cast<hipStream_t>(stream));
+  }
   if (int e = triteia_hip_route_plan(token_indices, index_offset, n_deltas, prob_n, workspace, workspace_bytes, dev, stream))
     return e;
   return triteia_hip_sbmm_2_4_planned(A, B, meta, C, s, workspace, n_deltas, prob_m, prob_n, prob_k, accumulate, dev, stream);
