@@ -1,0 +1,139 @@
+"""GPU tests at BASELINE's full sizes (configs 3 and 4), where a CPU dequantise of every delta would
+take minutes: size-independent properties plus a torch-on-GPU dequantise-then-matmul of sampled
+deltas (the torch codec is itself checked bit-exactly against the oracle in test_codec_cpu.py).
+
+  * routing: every sampled routed row equals, bit for bit, the single-matrix product of that row
+    alone with its own delta; rows with index -1 are exactly zero (or exactly the base output);
+  * exact scaling: out(2x) == 2 out(x) bit for bit wherever the output is a normal fp16 number
+    (powers of two commute with every rounding here);
+  * token-order invariance: permuting the batch permutes the output rows bit for bit;
+  * sampled deltas against fp32 matmul on their dequantised weights, relative Frobenius <= 2e-3.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from triteia_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from triteia_amd.python import ops as _ops
+    return _ops
+
+
+def _check_properties(ops, q, me, s, x, idx_np, sample_rows, sample_deltas, what):
+    from triteia_amd.python.ops.utils.sparsity import unpack_2_4
+    idx = torch.from_numpy(idx_np).to(DEV)
+    out = ops.sbmm_4bit_2_4_native(q, x, me, s, idx)
+    torch.cuda.synchronize()
+    assert bool((out[idx < 0] == 0).all()), f"{what}: -1 rows must stay zero"
+    for t in sample_rows:
+        d = int(idx_np[t])
+        if d >= 0:
+            alone = ops.matmul_4bit_2_4(q[d], x[t:t + 1], me[d], s[d])
+            assert torch.equal(alone[0], out[t]), f"{what}: row {t} differs from its own delta's product"
+    out2 = ops.sbmm_4bit_2_4_native(q, x * 2, me, s, idx)
+    normal = out.abs() >= 2.0 ** -13             # fp16 subnormals round differently after doubling
+    assert torch.equal(out2[normal], (out * 2)[normal]), f"{what}: out(2x) != 2 out(x)"
+    assert float((out2.float() - 2 * out.float()).abs().max()) <= 2.0 ** -23
+    perm = torch.randperm(x.shape[0], generator=torch.Generator().manual_seed(1)).to(DEV)
+    outp = ops.sbmm_4bit_2_4_native(q, x[perm].contiguous(), me, s, idx[perm].contiguous())
+    assert torch.equal(outp, out[perm]), f"{what}: token order changes the result"
+    for d in sample_deltas:
+        rows = torch.nonzero(idx == d).flatten()
+        if rows.numel() == 0:
+            continue
+        Wd = unpack_2_4(q[d], me[d], s[d]).float()
+        ref = x[rows].float() @ Wd
+        err = (out[rows].float() - ref).norm() / ref.norm()
+        assert float(err) <= 2e-3, f"{what}: delta {d} relative Frobenius error {float(err):.3e}"
+        del Wd
+    return out
+
+
+def test_config3_ldmm_shape(ops):
+    wl = W.config("cfg3")
+    say(wl.name)
+    q, me, s = W.random_packed_deltas(wl.n_deltas, wl.k, wl.m, wl.seed, DEV)
+    x = W.random_activations(wl.tokens, wl.k, wl.seed + 1, DEV)
+    used = np.unique(wl.indices[wl.indices >= 0])
+    out = _check_properties(ops, q, me, s, x, wl.indices, range(0, wl.tokens, 37), [int(used[0]), int(used[-1])], "cfg3 delta")
+    # the whole ldmm: base GEMM + LoRA (rank 16, 32 adapters, same routing) + delta
+    g = torch.Generator(device=DEV).manual_seed(7)
+    base = (torch.randn((wl.m, wl.k), generator=g, device=DEV) * 0.02).half()
+    A = (torch.randn((wl.n_lora, wl.k, wl.lora_rank), generator=g, device=DEV) * 0.01).half()
+    B = (torch.randn((wl.n_lora, wl.lora_rank, wl.m), generator=g, device=DEV) * 0.01).half()
+    idx = torch.from_numpy(wl.indices).to(DEV)
+    y_delta = ops.sbmm_4bit_2_4_native(q, x, me, s, idx, base_weight=base)
+    y0 = torch.matmul(x, base.t())
+    assert torch.equal(y_delta[idx < 0], y0[idx < 0])
+    err = ((y_delta.float() - y0.float()) - out.float()).norm() / out.float().norm()
+    assert float(err) < 5e-3                       # accumulate-in-place = base + delta up to fp16 rounding of the sum
+    lora = ops.lora_sgmv_routed(A, B, x, idx)
+    ref_rows = torch.nonzero(idx >= 0).flatten()[:8]
+    for t in ref_rows.tolist():
+        a = int(idx[t])
+        v = (x[t].float() @ A[a].float()).half().float()
+        ref = v @ B[a].float()
+        assert torch.allclose(lora[t].float(), ref, rtol=5e-3, atol=5e-3 * float(ref.abs().max()))
+    assert bool((lora[idx < 0] == 0).all())
+    # mixed index space of ldmm: adapters 0..31, deltas 32..63
+    mixed = torch.where(idx >= 0, idx + (torch.arange(wl.tokens, device=DEV) % 2).int() * wl.n_lora, idx)
+    y = ops.ldmm(mixed, x, A, B, q, me, s)
+    is_delta = mixed >= wl.n_lora
+    assert torch.equal(y[is_delta], out[is_delta])
+    is_lora = (mixed >= 0) & ~is_delta
+    assert torch.allclose(y[is_lora].float(), lora[is_lora].float(), rtol=5e-3, atol=1e-3)
+    assert bool((y[mixed < 0] == 0).all())
+
+
+@pytest.mark.parametrize("tokens", [1, 16, 64, 256, 1024])
+def test_config4_70b_shape(ops, tokens):
+    wl = W.config("cfg4", tokens)
+    say(wl.name)
+    q, me, s = _cfg4_weights(wl)
+    x = W.random_activations(wl.tokens, wl.k, wl.seed + 1, DEV)
+    used = np.unique(wl.indices[wl.indices >= 0])
+    step = max(1, tokens // 5)
+    _check_properties(ops, q, me, s, x, wl.indices, range(0, tokens, step), [int(used[0])], f"cfg4 T={tokens}")
+
+
+_CFG4 = {}
+
+
+def _cfg4_weights(wl):
+    # 64 deltas of 8192 x 28672 = 5.64 GB packed: built once for the five token counts
+    if "w" not in _CFG4:
+        _CFG4["w"] = W.random_packed_deltas(wl.n_deltas, wl.k, wl.m, wl.seed, DEV)
+    return _CFG4["w"]
+
+
+def test_bmm_many_tokens_per_matrix(ops):
+    say("bmm 3 x 150 tokens, 4096 x 4096 (wide tiles + narrow rest)")
+    from triteia_amd.python.ops.utils.sparsity import unpack_2_4
+    b, t, k, m = 3, 150, 4096, 4096
+    q, me, s = W.random_packed_deltas(b, k, m, 77, DEV)
+    x = W.random_activations(b * t, k, 78, DEV).reshape(b, t, k)
+    out = ops.bmm_4bit_2_4(q, x, me, s)
+    for i in range(b):
+        ref = x[i].float() @ unpack_2_4(q[i], me[i], s[i]).float()
+        err = (out[i].float() - ref).norm() / ref.norm()
+        assert float(err) <= 2e-3
+
+
+def test_reference_import_path_alias():
+    import triteia.python.ops as ref_ops
+    from triteia.python.capi import mul_2_4  # noqa: F401
+    from triteia.python.nn.linear import sparse_low_precision_linear  # noqa: F401
+    assert hasattr(ref_ops, "sbmm_4bit_2_4_native") and hasattr(ref_ops, "ldmm")
