@@ -131,47 +131,50 @@ __device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* 
 
 __device__ __forceinline__ int sgmv_row(const SgmvArgs& a, int i) { return a.perm ? a.perm[i] : i; }
 
-// wide -> narrow (d_out <= 128): grid (n_groups, row_tiles), block 256.
-// The flat weight [d_in * d_out] is read fully coalesced: thread t owns column
-// j = t % d_out of k rows t / d_out, t / d_out + 256 / d_out, ...
-template <int ROWS>
+// wide -> narrow (d_out <= DOUT <= 128): grid (n_groups, row slots), block 256; a block computes
+// one token row at a time.  Thread j takes the 8-row slabs j, j + 256, ... of the adapter matrix
+// (8 * d_out consecutive halfs, so a wavefront reads 64 slabs back to back) against 8 activations,
+// keeping d_out partial sums; the 256 partial vectors are then summed by shuffles and LDS.
+template <int DOUT>
 __global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgs a) {
-  __shared__ float part[ROWS][256];
+  __shared__ float part[4][DOUT];
   SgmvGroup g;
   if (!sgmv_group(a, blockIdx.x, &g)) return;
   const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
   const int dn = a.d_out;
-  const int kpar = 256 / dn;            // k rows covered per sweep (d_out divides 256 or threads idle)
-  const int j = tid % dn, ks = tid / dn;
-  const bool active = ks < kpar;
-  for (int r0 = blockIdx.y * ROWS; r0 < g.count; r0 += gridDim.y * ROWS) {
-    float acc[ROWS];
-    const _Float16* xr[ROWS];
+  for (int rr = blockIdx.y; rr < g.count; rr += gridDim.y) {
+    const int row = sgmv_row(a, g.start + rr);
+    const _Float16* x = a.x + (long)row * a.x_stride;
+    float acc[DOUT];
 #pragma unroll
-    for (int i = 0; i < ROWS; i++) {
-      acc[i] = 0.f;
-      xr[i] = (r0 + i < g.count) ? a.x + (long)sgmv_row(a, g.start + r0 + i) * a.x_stride : nullptr;
-    }
-    if (active) {
-      for (int k = ks; k < a.d_in; k += kpar) {
-        const float wv = (float)g.w[(long)k * dn + j];
+    for (int j = 0; j < DOUT; j++) acc[j] = 0.f;
+    for (int k0 = tid * 8; k0 < a.d_in; k0 += 256 * 8) {
+      const lhalf8_t xv = *reinterpret_cast<const lhalf8_t*>(x + k0);
+      const _Float16* wk = g.w + (long)k0 * dn;
 #pragma unroll
-        for (int i = 0; i < ROWS; i++)
-          if (xr[i]) acc[i] += wv * (float)xr[i][k];
+      for (int e = 0; e < 8; e++) {
+        const float xe = (float)xv[e];
+#pragma unroll
+        for (int j0 = 0; j0 < DOUT; j0 += 8) {
+          if (j0 < dn) {
+            const lhalf8_t wv = *reinterpret_cast<const lhalf8_t*>(wk + (long)e * dn + j0);
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[j0 + j] += xe * (float)wv[j];
+          }
+        }
       }
     }
 #pragma unroll
-    for (int i = 0; i < ROWS; i++) part[i][tid] = active ? acc[i] : 0.f;
+    for (int j = 0; j < DOUT; j++) {
+      const float v = wave_sum(acc[j]);
+      if (lane == 0) part[wave][j] = v;
+    }
     __syncthreads();
-    // thread t < ROWS * dn sums the kpar partials of (row t / dn, column t % dn)
-    for (int o = tid; o < ROWS * dn; o += 256) {
-      const int i = o / dn, jj = o % dn;
-      if (r0 + i < g.count) {
-        float s = 0.f;
-        for (int kk = 0; kk < kpar; kk++) s += part[i][kk * dn + jj];
-        _Float16* yp = a.y + (long)sgmv_row(a, g.start + r0 + i) * a.y_stride + jj;
-        *yp = (_Float16)((float)*yp + s * a.scale);
-      }
+    if (tid < dn) {
+      const float sum = part[0][tid] + part[1][tid] + part[2][tid] + part[3][tid];
+      _Float16* yp = a.y + (long)row * a.y_stride + tid;
+      *yp = (_Float16)((float)*yp + sum * a.scale);
     }
     __syncthreads();
   }
@@ -189,7 +192,7 @@ __global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgs a) {
   float w[DIN];
 #pragma unroll
   for (int i = 0; i < DIN; i++) w[i] = (ok && i < a.d_in) ? (float)g.w[(long)i * a.d_out + j] : 0.f;
-  for (int rr = 0; rr < g.count; rr++) {
+  for (int rr = blockIdx.z; rr < g.count; rr += gridDim.z) {
     const int row = sgmv_row(a, g.start + rr);
     __syncthreads();
     if (threadIdx.x < DIN) xs[threadIdx.x] = threadIdx.x < a.d_in ? (float)a.x[(long)row * a.x_stride + threadIdx.x] : 0.f;
@@ -201,6 +204,46 @@ __global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgs a) {
       _Float16* yp = a.y + (long)row * a.y_stride + j;
       *yp = (_Float16)((float)*yp + acc * a.scale);
     }
+  }
+}
+
+// narrow -> wide for d_in <= DIN <= 32: grid (n_groups, ceil(d_out / 2048), row slots), block 256.
+// A thread owns 8 consecutive output columns: its d_in x 8 weight patch stays in registers while
+// it walks the group's rows (16-byte loads and stores throughout, no barriers).
+template <int DIN>
+__global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgs a) {
+  SgmvGroup g;
+  if (!sgmv_group(a, blockIdx.x, &g)) return;
+  const int j0 = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (j0 >= a.d_out) return;
+  lhalf8_t w[DIN];
+#pragma unroll
+  for (int i = 0; i < DIN; i++) {
+    if (i < a.d_in) w[i] = *reinterpret_cast<const lhalf8_t*>(g.w + (long)i * a.d_out + j0);
+    else w[i] = lhalf8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+  for (int rr = blockIdx.z; rr < g.count; rr += gridDim.z) {
+    const int row = sgmv_row(a, g.start + rr);
+    const _Float16* xr = a.x + (long)row * a.x_stride;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] = 0.f;
+#pragma unroll
+    for (int i0 = 0; i0 < DIN; i0 += 8) {
+      if (i0 < a.d_in) {
+        const lhalf8_t xv = *reinterpret_cast<const lhalf8_t*>(xr + i0);   // same address in every lane
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) acc[e] += (float)xv[i] * (float)w[i0 + i][e];
+      }
+    }
+    _Float16* yp = a.y + (long)row * a.y_stride + j0;
+    const lhalf8_t old = *reinterpret_cast<const lhalf8_t*>(yp);
+    lhalf8_t o;
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = (_Float16)((float)old[e] + acc[e] * a.scale);
+    *reinterpret_cast<lhalf8_t*>(yp) = o;
   }
 }
 

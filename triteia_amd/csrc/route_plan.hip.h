@@ -29,6 +29,7 @@ constexpr int kPlanWideTile = 64;      // tokens per wide tile
 constexpr int kPlanWideMinRest = 33;   // a rest of at least this many tokens still forms a wide tile
 constexpr int kPlanMaxDeltas = 8192;  // per-delta cursors live in LDS
 constexpr int kPlanThreads = 256;
+constexpr int kPlanCachedTokens = 8192;  // token indices kept in LDS between the two passes
 constexpr int kPlanMinTile = 16;      // smallest tile size a plan can be built for
 
 struct PlanLayout {
@@ -72,6 +73,7 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
                                                                  int n_deltas, int index_offset, int tile, int wide,
                                                                  int* __restrict__ ws) {
   __shared__ int s_cursor[kPlanMaxDeltas];
+  __shared__ int s_delta[kPlanCachedTokens];   // pass 1 leaves each token's delta here for pass 2
   const PlanLayout L = plan_layout(n_tokens, n_deltas);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -79,8 +81,10 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
   for (int d = tid; d < n_deltas; d += kPlanThreads) s_cursor[d] = 0;
   __syncthreads();
   for (int t = tid; t < n_tokens; t += kPlanThreads) {
-    const int d = indices[t] - index_offset;
-    if (d >= 0 && d < n_deltas) atomicAdd(&s_cursor[d], 1);
+    int d = indices[t] - index_offset;
+    if (d < 0 || d >= n_deltas) d = -1;
+    if (t < kPlanCachedTokens) s_delta[t] = d;
+    if (d >= 0) atomicAdd(&s_cursor[d], 1);
   }
   __syncthreads();
 
@@ -135,21 +139,28 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
       const int t = base + lane;
       int d = -1;
       if (t < n_tokens) {
-        d = indices[t] - index_offset;
-        if (d < 0 || d >= n_deltas) d = -1;
+        if (t < kPlanCachedTokens) {
+          d = s_delta[t];
+        } else {
+          d = indices[t] - index_offset;
+          if (d < 0 || d >= n_deltas) d = -1;
+        }
       }
-      unsigned long long todo = __ballot(d >= 0);
-      while (todo) {
-        const int leader = __ffsll((long long)todo) - 1;
-        const int dl = __shfl(d, leader, 64);
-        const unsigned long long same = __ballot(d == dl) & todo;
-        const int first = s_cursor[dl];
-        if (d == dl && ((same >> lane) & 1ull)) ws[L.perm + first + __popcll(same & ((1ull << lane) - 1ull))] = t;
-        // every lane has read s_cursor[dl] before the leader bumps it
+      // lanes holding the same delta, found for all lanes at once: intersect, bit by bit of the
+      // delta id, the lanes that agree with this lane on that bit
+      const unsigned long long valid = __ballot(d >= 0);
+      unsigned long long same = valid;
+      for (int bit = 0; (1 << bit) < n_deltas; bit++) {
+        const unsigned long long set = __ballot((d >> bit) & 1);
+        same &= ((d >> bit) & 1) ? set : ~set;
+      }
+      if (d >= 0) {
+        const int rank = __popcll(same & ((1ull << lane) - 1ull));
+        const int first = s_cursor[d];
+        ws[L.perm + first + rank] = t;
+        // every lane of the group has read the cursor before its first lane moves it
         __builtin_amdgcn_wave_barrier();
-        if (lane == leader) s_cursor[dl] = first + __popcll(same);
-        __builtin_amdgcn_wave_barrier();
-        todo &= ~same;
+        if (rank == 0) s_cursor[d] = first + __popcll(same);
       }
     }
   }

@@ -374,15 +374,21 @@ static int launch_sgmv(SgmvArgs a, int max_rows, hipStream_t st) {
   if (a.d_in % 8 != 0 || a.d_out % 8 != 0 || narrow > kLoraMaxNarrow)
     return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "No suitable kernel. d_in=%d d_out=%d", a.d_in, a.d_out);
   if (a.n_groups <= 0) return TRITEIA_HIP_OK;
+  // rows of a group are spread over y (shrink) / z (expand); group sizes live on the device
+  int row_slots = max_rows < 64 ? max_rows : 64;
+  if (row_slots < 1) row_slots = 1;
   if (a.d_in >= a.d_out) {
-    int row_tiles = (max_rows + 3) / 4;
-    if (row_tiles > 64) row_tiles = 64;
-    if (row_tiles < 1) row_tiles = 1;
-    hipLaunchKernelGGL((sgmv_shrink_kernel<4>), dim3(a.n_groups, row_tiles), dim3(256), 0, st, a);
+    const dim3 grid(a.n_groups, row_slots);
+    if (a.d_out <= 16) hipLaunchKernelGGL((sgmv_shrink_kernel<16>), grid, dim3(256), 0, st, a);
+    else if (a.d_out <= 32) hipLaunchKernelGGL((sgmv_shrink_kernel<32>), grid, dim3(256), 0, st, a);
+    else if (a.d_out <= 64) hipLaunchKernelGGL((sgmv_shrink_kernel<64>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((sgmv_shrink_kernel<128>), grid, dim3(256), 0, st, a);
   } else {
-    const dim3 grid(a.n_groups, (a.d_out + 255) / 256);
-    if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_kernel<16>), grid, dim3(256), 0, st, a);
-    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_kernel<32>), grid, dim3(256), 0, st, a);
+    const int rz = row_slots < 8 ? row_slots : 8;
+    const dim3 grid(a.n_groups, (a.d_out + 255) / 256, rz);
+    const dim3 vgrid(a.n_groups, (a.d_out + 2047) / 2048, row_slots < 32 ? row_slots : 32);
+    if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_vec_kernel<16>), vgrid, dim3(256), 0, st, a);
+    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_vec_kernel<32>), vgrid, dim3(256), 0, st, a);
     else if (a.d_in <= 64) hipLaunchKernelGGL((sgmv_expand_kernel<64>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((sgmv_expand_kernel<128>), grid, dim3(256), 0, st, a);
   }
@@ -413,7 +419,7 @@ int triteia_hip_sgmv(void* y, const void* x, const void* w_ptrs, const void* s, 
   a.n_adapters = num_problems;
   a.scale = 1.0f;
   // segment lengths live on the device; size the row-tile dimension for a few rows per segment
-  return launch_sgmv(a, 16, static_cast<hipStream_t>(stream));
+  return launch_sgmv(a, 64, static_cast<hipStream_t>(stream));
 }
 
 int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
