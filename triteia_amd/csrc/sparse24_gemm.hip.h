@@ -95,16 +95,24 @@ struct Sparse24Args {
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
 __device__ __forceinline__ half2_t bits_h2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 
+// (w & mask) | 0x64006400 in one instruction: a bitfield insert of w's masked bits into the fp16
+// pair (1024, 1024).  (The compiler would emit an AND and an OR: VOP3 takes no two literals.)
+__device__ __forceinline__ uint32_t insert_into_1024(uint32_t w, uint32_t mask) {
+  uint32_t r;
+  const uint32_t magic = 0x64006400u;
+  asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(r) : "s"(mask), "v"(w), "v"(magic));
+  return r;
+}
 // nibbles 0 and 4 of w -> (n0 - 8, n4 - 8)
 __device__ __forceinline__ uint32_t dequant_even(uint32_t w) {
   const half2_t bias = {(_Float16)1032.0f, (_Float16)1032.0f};
-  return h2_bits(bits_h2((w & 0x000f000fu) | 0x64006400u) - bias);
+  return h2_bits(bits_h2(insert_into_1024(w, 0x000f000fu)) - bias);
 }
 // nibbles 1 and 5 of w -> (n1 - 8, n5 - 8):  (1024 + 16 n) / 16 - 72
 __device__ __forceinline__ uint32_t dequant_odd(uint32_t w) {
   const half2_t mul = {(_Float16)0.0625f, (_Float16)0.0625f};
   const half2_t add = {(_Float16)-72.0f, (_Float16)-72.0f};
-  return h2_bits(bits_h2((w & 0x00f000f0u) | 0x64006400u) * mul + add);
+  return h2_bits(bits_h2(insert_into_1024(w, 0x00f000f0u)) * mul + add);
 }
 
 // Workgroup barrier that orders LDS traffic only: outstanding global loads (the prefetch
@@ -327,7 +335,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 // NT = widest token tile (16*NT tokens per pass) the instantiation supports; narrower passes
 // take the cheaper code path (fewer activation loads and MFMAs) at the same register budget.
 template <int NT, int KW, int DEPTH>
-__global__ __launch_bounds__(64 * KW) void sparse24_grouped_kernel(const Sparse24Args p) {
+__global__ __launch_bounds__(64 * KW, (NT == 1 ? 3 : (NT == 2 ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
   __shared__ float red[KW][16][kRedStride];
   __shared__ int s_rows[16 * NT];
 

@@ -82,8 +82,9 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   if (tsplit > 65535) tsplit = 65535;
   const long cb_pad = (a.m / 128 + 7) / 8 * 8;   // column blocks padded to the 8 XCDs
   const int kw = env_int("TRITEIA_HIP_KW", 4);
-  // register budget: two steps in flight for the narrow tiles, one for the 64-token tile
-  const int depth = env_int("TRITEIA_HIP_DEPTH", nt == 4 ? 1 : 2);
+  // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight, the
+  // 32-token kernel 2 per CU with two, the 64-token kernel 1 per CU with one
+  const int depth = env_int("TRITEIA_HIP_DEPTH", nt == 2 ? 2 : 1);
   const long units = (long)a.n_groups * cb_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   const dim3 grid((unsigned)units, (unsigned)tsplit);
