@@ -58,6 +58,35 @@ def test_matmul_4bit_2_4(ops, n, k, m, seed):
     check_close(out, ref, what="matmul_4bit_2_4")
 
 
+@pytest.mark.parametrize("kernel", ["wide64", "wide128"])
+@pytest.mark.parametrize("n,k,m,seed", [
+    (64, 128, 512, 21), (128, 128, 512, 22), (128, 256, 128, 23),      # one tile, 1 and 2 k steps
+    (200, 384, 384, 24), (321, 512, 640, 25), (130, 640, 256, 26),     # ragged tokens, partial column groups
+    (256, 1024, 1024, 27), (448, 896, 1152, 28),                       # 7 k steps: every ring phase
+    (192, 192, 256, 29),                                               # k = 64 (mod 128): falls back to the narrow kernel
+])
+def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
+    """The matrix-core-bound kernels (64- and 128-token tiles), forced onto small ragged
+    shapes that the launcher would give to the narrow kernel."""
+    say(f"matmul {kernel} n={n} k={k} m={m} seed={seed}")
+    monkeypatch.setenv("TRITEIA_HIP_WIDE_MIN_UNITS", "1")
+    monkeypatch.setenv("TRITEIA_HIP_WIDE128_MIN_UNITS", "1")
+    monkeypatch.setenv("TRITEIA_HIP_WIDE128", "1" if kernel == "wide128" else "0")
+    qw, meta, s = make_deltas(1, k, m, seed)
+    x = activations(n, k, seed + 1)
+    ref = orc.matmul_4bit_2_4(qw[0], x, meta[0], s[0])
+    gq, gm, gs, gx = to_gpu(qw[0], meta[0], s[0], x)
+    out = ops.matmul_4bit_2_4(gq, gx, gm, gs)
+    torch.cuda.synchronize()
+    check_close(out, ref, what=f"matmul_4bit_2_4 {kernel}")
+    # same inputs through the narrow kernel: equal up to the order of fp32 accumulation
+    monkeypatch.setenv("TRITEIA_HIP_WIDE", "0")
+    narrow = ops.matmul_4bit_2_4(gq, gx, gm, gs)
+    torch.cuda.synchronize()
+    rel = ((out.float() - narrow.float()).norm() / narrow.float().norm()).item()
+    assert rel < 1e-4, rel
+
+
 def test_matmul_many_tokens_reference_test_shape(ops):
     # the reference's own test shape m = n = k = 4096 (tests/ops/test_matmul.py:30)
     n = k = m = 4096

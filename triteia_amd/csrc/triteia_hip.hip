@@ -13,6 +13,7 @@
 #include "route_plan.hip.h"
 #include "sparse24_gemm.hip.h"
 #include "sparse24_wide.hip.h"
+#include "sparse24_wide128.hip.h"
 
 namespace {
 
@@ -146,31 +147,66 @@ int launch_wide(const Sparse24Args& a, hipStream_t st) {
   return check_launch("sparse24_wide_kernel");
 }
 
-// The wide kernel pays off when there are enough 64-token x 512-column tiles to occupy the
-// GPU; below that the narrow kernel's smaller units win.  TRITEIA_HIP_WIDE=0 disables it.
-bool wide_enabled() { return env_int("TRITEIA_HIP_WIDE", 1) != 0; }
-constexpr long kWideMinUnits = 128;
+// 128-token x 512-column tiles (one workgroup per CU, 128.5 KB of dynamic LDS).
+int launch_wide128(const Sparse24Args& a, hipStream_t st) {
+  if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
+  const long cgs = (a.m / 128 + 3) / 4;
+  const long cg_pad = (cgs + 7) / 8 * 8;
+  const long chunks = a.tiles ? 1 : (a.uniform_count + kWide128Tokens - 1) / kWide128Tokens;
+  const long units = (long)a.n_groups * chunks * cg_pad;
+  if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
+  // the attribute is per device; setting it again is cheap and keeps the library free of global state
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse24_wide128_kernel),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kWide128LdsBytes) != hipSuccess)
+    return fail(TRITEIA_HIP_ERR_RUNTIME, "sparse24_wide128_kernel: cannot reserve %d bytes of LDS", kWide128LdsBytes);
+  Sparse24Args b = a;
+  if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
+  hipLaunchKernelGGL(sparse24_wide128_kernel, dim3((unsigned)units), dim3(256), kWide128LdsBytes, st, b);
+  return check_launch("sparse24_wide128_kernel");
+}
 
-// `tokens` rows per group, `stride` rows between groups: full 64-token chunks (and a rest above
-// 32 tokens) go to the wide kernel, what is left to the narrow one.
+// The wide kernels pay off when there are enough tiles to occupy the GPU; below that the
+// narrow kernel's smaller units win.  TRITEIA_HIP_WIDE=0 disables both, TRITEIA_HIP_WIDE128=0
+// the 128-token one; TRITEIA_HIP_WIDE_MIN_UNITS / TRITEIA_HIP_WIDE128_MIN_UNITS move the thresholds.
+bool wide_enabled() { return env_int("TRITEIA_HIP_WIDE", 1) != 0; }
+bool wide128_enabled() { return wide_enabled() && env_int("TRITEIA_HIP_WIDE128", 1) != 0; }
+constexpr long kWideMinUnits = 128;
+constexpr long kWide128MinUnits = 192;
+
+// `tokens` rows per group, `stride` rows between groups: the head of each group goes to the
+// 128-token kernel, then to the 64-token kernel (full tiles, and a rest above half a tile),
+// what is left to the narrow one.
 int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n_groups, hipStream_t st) {
   a.n_groups = n_groups;
   a.uniform_stride = stride;
   a.delta_step = delta_step;
-  int wide_tokens = 0;
   const long cgs = (a.m / 128 + 3) / 4;
-  if (wide_enabled() && a.k % 128 == 0 && (long)n_groups * (tokens / kWideTokens) * cgs >= kWideMinUnits) {
-    wide_tokens = tokens / kWideTokens * kWideTokens;
-    if (tokens - wide_tokens >= kPlanWideMinRest) wide_tokens = tokens;
-  }
-  if (wide_tokens > 0) {
+  int done = 0;
+  // (the 128-token kernel addresses activations with 32-bit byte offsets)
+  const bool x_below_4g = ((long)(n_groups - 1) * stride + tokens) * a.x_stride * 2 < (1L << 32);
+  if (wide128_enabled() && a.k % 128 == 0 && x_below_4g &&
+      (long)n_groups * (tokens / kWide128Tokens) * cgs >= env_int("TRITEIA_HIP_WIDE128_MIN_UNITS", kWide128MinUnits)) {
+    int t = tokens / kWide128Tokens * kWide128Tokens;
+    if (tokens - t > kWideTokens) t = tokens;
     a.uniform_first = 0;
-    a.uniform_count = wide_tokens;
-    if (int e = launch_wide(a, st)) return e;
+    a.uniform_count = t;
+    if (int e = launch_wide128(a, st)) return e;
+    done = t;
   }
-  const int rest = tokens - wide_tokens;
+  int rest = tokens - done;
+  if (rest > 0 && wide_enabled() && a.k % 128 == 0 &&
+      (done > 0 ? rest >= kPlanWideMinRest
+                : (long)n_groups * (rest / kWideTokens) * cgs >= env_int("TRITEIA_HIP_WIDE_MIN_UNITS", kWideMinUnits))) {
+    int t = rest / kWideTokens * kWideTokens;
+    if (rest - t >= kPlanWideMinRest) t = rest;
+    a.uniform_first = done;
+    a.uniform_count = t;
+    if (int e = launch_wide(a, st)) return e;
+    done += t;
+  }
+  rest = tokens - done;
   if (rest > 0) {
-    a.uniform_first = wide_tokens;
+    a.uniform_first = done;
     a.uniform_count = rest;
     const int nt = pick_nt(rest, 1);
     return launch_sparse24(a, nt, (rest + 16 * nt - 1) / (16 * nt), st);
