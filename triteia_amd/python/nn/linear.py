@@ -55,3 +55,56 @@ class sparse_low_precision_linear(nn.Module):
         self.qweight.copy_(qweight)
         self.meta.copy_(meta)
         self.scale.copy_(s16)
+
+
+class multi_delta_linear(nn.Module):
+    """One linear layer serving many fine-tuned variants of a base model at once: an optional
+    dense fp16 base weight plus `n_deltas` stacked 2:4 int4 deltas; every token picks its delta
+    (or none, index -1) through an index vector.  The layer a serving engine calls once per
+    projection (the reference has the op, ops/matmul/sbmm.py:89-142, but no module around it).
+
+    Buffers: qweight int32 [N, k/32, 2m], meta int16 [N, m, k/16], scale fp16 [N, 1, m],
+    base fp16 [m, k] (optional).  `forward(x, indices)` routes on the device; with
+    `plan=route_plan(indices, N)` the same routing is shared by all layers of a forward pass."""
+
+    def __init__(self, infeatures, outfeatures, n_deltas, with_base=False):
+        super().__init__()
+        assert infeatures % 128 == 0, f"Input features must be a multiple of 128, got {infeatures}"
+        assert outfeatures % 256 == 0, f"Output features must be a multiple of 256, got {outfeatures}"
+        self.infeatures, self.outfeatures, self.n_deltas = infeatures, outfeatures, n_deltas
+        self.register_buffer("qweight", torch.zeros((n_deltas, infeatures // 32, outfeatures * 2), dtype=torch.int32))
+        self.register_buffer("meta", torch.zeros((n_deltas, outfeatures, infeatures // 16), dtype=torch.int16))
+        self.register_buffer("scale", torch.zeros((n_deltas, 1, outfeatures), dtype=torch.float16))
+        self.register_buffer("base", torch.zeros((outfeatures, infeatures), dtype=torch.float16) if with_base else None)
+
+    @torch.no_grad()
+    def load_delta(self, i, module_or_qweight, meta=None, scale=None):
+        """Copy one packed delta into slot i: from a `sparse_low_precision_linear` or from its three tensors."""
+        if isinstance(module_or_qweight, sparse_low_precision_linear):
+            m = module_or_qweight
+            module_or_qweight, meta, scale = m.qweight, m.meta, m.scale
+        self.qweight[i].copy_(module_or_qweight)
+        self.meta[i].copy_(meta)
+        self.scale[i].copy_(scale.reshape(1, -1))
+
+    @torch.no_grad()
+    def pack_delta(self, i, weight, scales):
+        """Quantise and pack a dense [k, m] fp16 delta with per-column scales into slot i."""
+        layer = sparse_low_precision_linear(self.infeatures, self.outfeatures).to(self.qweight.device)
+        layer.pack(weight, scales)
+        self.load_delta(i, layer)
+
+    def forward(self, x, indices, plan=None):
+        """x [..., k] fp16, indices int32 [tokens] in {-1, 0..N-1} (any order) -> [..., m]."""
+        from triteia_amd.python.capi import sbmm_2_4_planned, sbmm_2_4_routed
+        x2 = x.reshape(-1, x.shape[-1])
+        x2 = x2 if x2.is_contiguous() else x2.contiguous()
+        if self.base is not None:
+            y = torch.matmul(x2, self.base.t())
+        else:
+            y = torch.zeros((x2.shape[0], self.outfeatures), dtype=x.dtype, device=x.device)
+        if plan is not None:
+            sbmm_2_4_planned(x2, self.qweight, self.meta, y, self.scale, plan, accumulate=True)
+        else:
+            sbmm_2_4_routed(x2, self.qweight, self.meta, y, self.scale, indices.to(torch.int32), accumulate=True)
+        return y.view(x.shape[:-1] + (self.outfeatures,))

@@ -91,7 +91,8 @@ class Workload:
 def config(name, tokens=None):
     """The five benchmark configurations (seed = 1000 + index)."""
     if name == "cfg0":
-        return Workload("cfg0 matmul_4bit_2_4 x[16,4096] W[4096x4096]", "matmul", 4096, 4096, 1, 16, 1000)
+        t = 16 if tokens is None else tokens
+        return Workload(f"cfg0 matmul_4bit_2_4 x[{t},4096] W[4096x4096]", "matmul", 4096, 4096, 1, t, 1000)
     if name == "cfg1":
         return Workload("cfg1 bmm_4bit_2_4 8 deltas 4096x4096, 1 token each", "bmm", 4096, 4096, 8, 8, 1001)
     if name == "cfg2":
