@@ -230,6 +230,42 @@ def test_sbmm_variants(ops, kind, T, N, m, k, sort, seed):
             assert torch.equal(multi, native) and torch.equal(runs, native)
 
 
+@pytest.mark.parametrize("T,N,used,seed", [
+    (64, 16, [0, 3, 5, 15], 41),        # most deltas without tokens: their prefetched weights are dropped
+    (64, 8, list(range(8)), 42),         # every delta in use, some with more than one 16-token pass
+    (33, 4, [2], 43),                    # one delta, three passes of 16 tokens at most (tile of 32)
+    (40, 64, [7, 63], 44),               # fewer than two tokens per delta: routes first, then requests
+])
+def test_fused_routing_static_groups(ops, monkeypatch, T, N, used, seed):
+    """Batches of at most 64 tokens are routed inside the multiply kernel; with at least two tokens per
+    delta every delta is a group of its own and its first weights are requested before the indices
+    have arrived.  Same bits as routing first (TRITEIA_HIP_EAGER=0) and as the plan-based path."""
+    say(f"fused routing T={T} N={N} used={used} seed={seed}")
+    k, m = 512, 384
+    qw, meta, s = make_deltas(N, k, m, seed)
+    x = activations(T, k, seed + 1)
+    rng = np.random.default_rng(seed + 2)
+    idx = rng.choice(np.array(used + [-1], dtype=np.int32), size=T).astype(np.int32)
+    ref = orc.sbmm_4bit_2_4(qw, x, meta, s, idx)
+    gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
+    outs = {}
+    for name, env in (("eager", {"TRITEIA_HIP_EAGER": "1"}), ("route-first", {"TRITEIA_HIP_EAGER": "0"}),
+                      ("planned", {"TRITEIA_HIP_FUSED_ROUTE": "0"})):
+        for key in ("TRITEIA_HIP_EAGER", "TRITEIA_HIP_FUSED_ROUTE"):
+            monkeypatch.delenv(key, raising=False)
+        for key, value in env.items():
+            monkeypatch.setenv(key, value)
+        out = torch.full((T, m), 3.0, dtype=torch.float16, device=DEV)      # rows without a delta must stay as they are
+        from triteia_amd.python.capi import sbmm_2_4_routed
+        sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
+        torch.cuda.synchronize()
+        outs[name] = out
+    none = torch.from_numpy(idx < 0).to(DEV)
+    assert bool((outs["eager"][none] == 3.0).all())
+    check_close(torch.where(none[:, None], torch.zeros_like(outs["eager"]), outs["eager"]), ref, what="fused routing")
+    assert torch.equal(outs["eager"], outs["route-first"]) and torch.equal(outs["eager"], outs["planned"])
+
+
 def test_sbmm_with_base_weight_accumulates_in_place(ops):
     say("sbmm with base weight")
     T, N, k, m = 24, 4, 256, 256

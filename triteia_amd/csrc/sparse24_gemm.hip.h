@@ -86,6 +86,7 @@ struct Sparse24Args {
   int delta_step;
   int n_deltas;             // deltas with index outside [0, n_deltas) are skipped
   int accumulate;           // 0: out = result, 1: out += result
+  int raw_static;           // fused routing with group g = delta g: weights are requested before the indices arrive
   int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run
 #ifdef TRITEIA_HIP_TIMELINE
   long long* timeline;      // [unit][wave][4] 100 MHz timestamps (debug builds only)
@@ -115,6 +116,18 @@ __device__ __forceinline__ uint32_t dequant_odd(uint32_t w) {
   return h2_bits(bits_h2(insert_into_1024(w, 0x00f000f0u)) * mul + add);
 }
 
+// fp16(old + acc * scale) with every step rounded on its own (fp32 product, fp32 sum, then fp16), and
+// the same expression whether or not there is an `old` to add to (0 otherwise).  Left to itself
+// the compiler fuses some instances of this into a single-rounding mixed-precision fma and not
+// others, so that the same row could differ in its last bit between two builds of the kernel
+// (token-tile sizes, accumulate or not); results must not depend on which kernel ran.
+__device__ __forceinline__ _Float16 scaled_sum_f16(_Float16 old, float acc, _Float16 scale) {
+#pragma clang fp contract(off)
+  const float prod = acc * (float)scale;
+  const float sum = (float)old + prod;
+  return (_Float16)sum;
+}
+
 // Workgroup barrier that orders LDS traffic only: outstanding global loads (the prefetch
 // ring) are not waited for.
 __device__ __forceinline__ void lds_barrier() {
@@ -131,6 +144,12 @@ struct StepFrag {
   uint4_t xb[NT][2];    // B slots 8..15 for u = 0, 1
 };
 
+// weights and metadata of one step, requested ahead of a tile pass
+struct WPre {
+  uint4_t wq[4];
+  uint4_t mt[2];
+};
+
 constexpr int kRedStride = 132;  // floats per token row in the reduction buffer (128 + pad)
 
 // Everything one workgroup knows about its (group, column block) before touching tokens.
@@ -143,6 +162,7 @@ struct TileCtx {
   int cb;                   // column block
   int tid, wave, lane, r, q;
   int raw_list;             // fused routing: lane s holds the token row of slot s of the group
+  half8_t sv;               // scales of this thread's 8 output features (requested at start-up)
 #ifdef TRITEIA_HIP_TIMELINE
   long long ts[4];          // debug builds: entry, operands requested, K loop done, end
 #endif
@@ -150,9 +170,10 @@ struct TileCtx {
 
 // One pass over K for up to 16*NTT tokens of one group: loads, sparse MFMAs, cross-wave
 // reduction, scaled fp16 store.  `first` = index of the pass's first token in the group's list.
-template <int NTT, int KW, int DEPTH>
+// USE_PRE: the weights of this wave's first step are already on their way in `pre`.
+template <int NTT, int KW, int DEPTH, bool USE_PRE = false>
 __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int first, int cnt,
-                                          float (*red)[16][kRedStride], int* s_rows) {
+                                          float (*red)[16][kRedStride], int* s_rows, const WPre* pre = nullptr) {
   const int r = c.r, q = c.q, wave = c.wave;
   const int k_rows = c.k_rows, n_steps = c.n_steps;
 
@@ -181,7 +202,16 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   }
   StepFrag<NTT> ring[DEPTH];
 #pragma unroll
-  for (int j = 0; j < DEPTH; j++) load_w(ring[j], wave + j * KW);
+  for (int j = 0; j < DEPTH; j++) {
+    if (USE_PRE && j == 0) {
+#pragma unroll
+      for (int a = 0; a < 4; a++) ring[0].wq[a] = pre->wq[a];
+      ring[0].mt[0] = pre->mt[0];
+      ring[0].mt[1] = pre->mt[1];
+    } else {
+      load_w(ring[j], wave + j * KW);
+    }
+  }
 
   // Every lane always loads from a valid address, so that the number of loads per step is
   // fixed and the hardware load counter can be waited on exactly (the output columns of the
@@ -316,17 +346,13 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 #pragma unroll
         for (int i = 0; i < 4; i++) { v[i] += a0[i]; v[4 + i] += a1[i]; }
       }
-      const half8_t sv = *reinterpret_cast<const half8_t*>(c.sc + f0);
+      const half8_t sv = c.sv;   // f0 is the same for every chunk of a thread: 64 * KW is a multiple of 16
       _Float16* op = p.out + (long)row * p.out_stride + c.cb * 128 + f0;
+      half8_t old = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (p.accumulate) old = *reinterpret_cast<const half8_t*>(op);
       half8_t o;
-      if (p.accumulate) {
-        const half8_t old = *reinterpret_cast<const half8_t*>(op);
 #pragma unroll
-        for (int i = 0; i < 8; i++) o[i] = (_Float16)((float)old[i] + v[i] * (float)sv[i]);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; i++) o[i] = (_Float16)(v[i] * (float)sv[i]);
-      }
+      for (int i = 0; i < 8; i++) o[i] = scaled_sum_f16(old[i], v[i], sv[i]);
       *reinterpret_cast<half8_t*>(op) = o;
     }
   }
@@ -334,7 +360,9 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 
 // NT = widest token tile (16*NT tokens per pass) the instantiation supports; narrower passes
 // take the cheaper code path (fewer activation loads and MFMAs) at the same register budget.
-template <int NT, int KW, int DEPTH>
+// EAGER: fused routing with group g = delta g (Sparse24Args::raw_static): the weights of the first
+// step are requested at once, together with the indices, instead of one memory round trip later.
+template <int NT, int KW, int DEPTH, bool EAGER = false>
 __global__ __launch_bounds__(64 * KW, (NT == 1 ? 3 : (NT == 2 ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
   __shared__ float red[KW][16][kRedStride];
   __shared__ int s_rows[16 * NT];
@@ -352,39 +380,78 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? 3 : (NT == 2 ? 2 : 1))) void sp
   const int i = unit - grp * cb_pad;
   const int cb = p.xcd_swizzle ? (i & 7) * (cb_pad >> 3) + (i >> 3) : i;
   if (cb >= col_blocks) return;
+
+  TileCtx c;
+  c.tid = threadIdx.x;
+  c.wave = c.tid >> 6;
+  c.lane = c.tid & 63;
+  c.r = c.lane & 15;
+  c.q = c.lane >> 4;
+  c.cb = cb;
+  c.raw_list = 0;
+  c.k_rows = p.k >> 5;                 // packed rows (32 dense k each)
+  c.n_steps = (c.k_rows + 3) >> 2;     // 128 dense k per step
+  c.qrow = p.m >> 1;
+  c.mrow = p.m >> 2;
+  // everything that depends on the delta: operand pointers and the request for this thread's scales
+  auto bind_delta = [&](int delta) {
+    c.qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * c.r;
+    c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.r >> 3)) * 16 + (c.r & 7);
+    c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;
+    c.sv = *reinterpret_cast<const half8_t*>(c.sc + (c.tid & 15) * 8);
+  };
+
   // group descriptor and live group count are fetched side by side (no dependent chain);
   // grp < p.n_groups (the host's upper bound) keeps the descriptor reads in bounds
   int delta, start, count;
-  int raw_list = 0;
+  WPre pre;
   if (p.raw_indices) {
     // Fused routing for small batches: every wavefront looks at all (<= 64) indices, one per
-    // lane, and works out the grp-th delta in use and the rows routed to it -- a few dozen
-    // instructions instead of a separate routing launch and a dependent descriptor read.
-    const int lane_ = threadIdx.x & 63;
+    // lane, and works out its delta and the rows routed to it -- a few dozen instructions
+    // instead of a separate routing launch and a dependent descriptor read.
     int d = -1;
-    if (lane_ < p.raw_count) {
-      d = p.raw_indices[lane_] - p.raw_offset;
-      if (d < 0 || d >= p.n_deltas) d = -1;
-    }
-    unsigned long long used = d >= 0 ? (1ull << d) : 0ull;
+    if (c.lane < p.raw_count) d = p.raw_indices[c.lane];
+    if (EAGER) {
+      // group g is delta g: its first weights are requested right behind the indices
+      if (grp >= p.n_deltas) return;
+      delta = grp;
+      bind_delta(delta);
+      const int tr = min((c.wave << 2) + c.q, c.k_rows - 1);
+      const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
+      const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const unsigned lo = __shfl_xor((unsigned)used, off, 64);
-      const unsigned hi = __shfl_xor((unsigned)(used >> 32), off, 64);
-      used |= ((unsigned long long)hi << 32) | lo;
+      for (int a = 0; a < 4; a++) pre.wq[a] = wp[a];
+      pre.mt[0] = mp[0];
+      pre.mt[1] = mp[8];
     }
-    if (grp >= __popcll(used)) return;
-    const unsigned long long below = (1ull << lane_) - 1ull;
-    const bool is_grp = ((used >> lane_) & 1ull) && __popcll(used & below) == grp;
-    delta = __ffsll((long long)__ballot(is_grp)) - 1;
+    d -= p.raw_offset;
+    if (c.lane >= p.raw_count || d < 0 || d >= p.n_deltas) d = -1;
+    const unsigned long long below = (1ull << c.lane) - 1ull;
+    if (!EAGER) {
+      // the grp-th delta in use
+      unsigned long long used = d >= 0 ? (1ull << d) : 0ull;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const unsigned lo = __shfl_xor((unsigned)used, off, 64);
+        const unsigned hi = __shfl_xor((unsigned)(used >> 32), off, 64);
+        used |= ((unsigned long long)hi << 32) | lo;
+      }
+      if (grp >= __popcll(used)) return;
+      const bool is_grp = ((used >> c.lane) & 1ull) && __popcll(used & below) == grp;
+      delta = __ffsll((long long)__ballot(is_grp)) - 1;
+    }
     const unsigned long long members = __ballot(d == delta);
     count = __popcll(members);
     start = 0;
     // slot s of the group = the s-th member token: a full permutation sends every member's
     // token id to the lane of its rank (non-members fill the lanes after the members)
     const int rank = __popcll(members & below);
-    const int dest = (d == delta) ? rank : count + (lane_ - rank);
-    raw_list = __builtin_amdgcn_ds_permute(dest << 2, lane_);
+    const int dest = (d == delta) ? rank : count + (c.lane - rank);
+    c.raw_list = __builtin_amdgcn_ds_permute(dest << 2, c.lane);
+    if (EAGER && count <= 0) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): let the requested weights land before the wave ends
+      return;
+    }
   } else if (p.tiles) {
     const int4 d = p.tiles[grp];
     delta = d.x;
@@ -399,36 +466,33 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? 3 : (NT == 2 ? 2 : 1))) void sp
     start = grp * p.uniform_stride + p.uniform_first;
     count = p.uniform_count;
   }
-  const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
-  if (grp >= n_groups) return;
-  if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
-
-  TileCtx c;
-  c.tid = threadIdx.x;
-  c.wave = c.tid >> 6;
-  c.lane = c.tid & 63;
-  c.r = c.lane & 15;
-  c.q = c.lane >> 4;
-  c.cb = cb;
-  c.raw_list = raw_list;
-  c.k_rows = p.k >> 5;                 // packed rows (32 dense k each)
-  c.n_steps = (c.k_rows + 3) >> 2;     // 128 dense k per step
-  c.qrow = p.m >> 1;
-  c.mrow = p.m >> 2;
-  c.qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * c.r;
-  c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.r >> 3)) * 16 + (c.r & 7);
-  c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;
+  if (!EAGER) {
+    const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
+    if (grp >= n_groups) return;
+    if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
+    bind_delta(delta);
+  }
 
   // blockIdx.y splits a group's tokens between workgroups (each re-streams the weights)
+  bool first_pass = true;
   for (int t0 = blockIdx.y * 16 * NT; t0 < count; t0 += gridDim.y * 16 * NT) {
     const int cnt = min(count - t0, 16 * NT);
-    if (NT == 1 || cnt <= 16) {
+    if (EAGER && first_pass) {
+      if (NT == 1 || cnt <= 16) {
+        tile_pass<1, KW, (NT == 1 ? DEPTH : 2), true>(p, c, start + t0, cnt, red, s_rows, &pre);
+      } else if (NT == 2 || cnt <= 32) {
+        tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), true>(p, c, start + t0, cnt, red, s_rows, &pre);
+      } else {
+        tile_pass<NT, KW, DEPTH, true>(p, c, start + t0, cnt, red, s_rows, &pre);
+      }
+    } else if (NT == 1 || cnt <= 16) {
       tile_pass<1, KW, (NT == 1 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);
     } else if (NT == 2 || cnt <= 32) {
       tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);
     } else {
       tile_pass<NT, KW, DEPTH>(p, c, start + t0, cnt, red, s_rows);
     }
+    first_pass = false;
     // the next pass over this group's tokens reuses s_rows / red
     if (t0 + gridDim.y * 16 * NT < count) lds_barrier();
   }

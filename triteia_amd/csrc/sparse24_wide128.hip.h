@@ -256,15 +256,11 @@ __global__ __launch_bounds__(256, 1) void sparse24_wide128_kernel(const Sparse24
     _Float16* op = p.out + (long)s_rows[slot] * p.out_stride + cb * 128 + 32 * q;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
+      half8_t old = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (p.accumulate) old = *reinterpret_cast<const half8_t*>(op + 8 * j);
       half8_t o;
-      if (p.accumulate) {
-        const half8_t old = *reinterpret_cast<const half8_t*>(op + 8 * j);
 #pragma unroll
-        for (int cc = 0; cc < 8; cc++) o[cc] = (_Float16)((float)old[cc] + acc[cc][nt][j] * (float)sv[j][cc]);
-      } else {
-#pragma unroll
-        for (int cc = 0; cc < 8; cc++) o[cc] = (_Float16)(acc[cc][nt][j] * (float)sv[j][cc]);
-      }
+      for (int cc = 0; cc < 8; cc++) o[cc] = scaled_sum_f16(old[cc], acc[cc][nt][j], sv[j][cc]);
       *reinterpret_cast<half8_t*>(op + 8 * j) = o;
     }
   }

@@ -70,9 +70,9 @@ int pick_nt(long tokens, long groups) {
   return 4;
 }
 
-template <int NT, int KW, int DEPTH>
+template <int NT, int KW, int DEPTH, bool EAGER = false>
 void launch_one(const Sparse24Args& a, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((sparse24_grouped_kernel<NT, KW, DEPTH>), grid, dim3(64 * KW), 0, st, a);
+  hipLaunchKernelGGL((sparse24_grouped_kernel<NT, KW, DEPTH, EAGER>), grid, dim3(64 * KW), 0, st, a);
 }
 
 // `nt`: token tile class; `tsplit`: workgroups along y sharing one group's tokens (run-table form
@@ -85,15 +85,25 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   const int kw = env_int("TRITEIA_HIP_KW", 4);
   // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight, the
   // 32-token kernel 2 per CU with two, the 64-token kernel 1 per CU with one
-  const int depth = env_int("TRITEIA_HIP_DEPTH", nt == 2 ? 2 : 1);
+  // (the eager form of fused routing holds one more step of weights: one step in flight for every tile)
+  const int depth = env_int("TRITEIA_HIP_DEPTH", nt == 2 && !(a.raw_indices && a.raw_static) ? 2 : 1);
+  if (a.raw_indices && a.raw_static && !(kw == 4 && depth == 1)) {
+    a.raw_static = 0;   // no eager build of this variant: route first, then request
+    a.n_groups = a.raw_count < a.n_deltas ? a.raw_count : a.n_deltas;
+  }
   const long units = (long)a.n_groups * cb_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   const dim3 grid((unsigned)units, (unsigned)tsplit);
 #define TRY(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
-  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 2)
+#define TRY_EAGER(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_, true>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
+  if (a.raw_indices && a.raw_static) {
+    TRY_EAGER(1, 4, 1) TRY_EAGER(2, 4, 1) TRY_EAGER(4, 4, 1)
+  }
+  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 2) TRY(1, 16, 1)
   TRY(2, 4, 1) TRY(2, 4, 2) TRY(2, 8, 1)
   TRY(4, 4, 1)
 #undef TRY
+#undef TRY_EAGER
   return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "no kernel variant for NT=%d KW=%d DEPTH=%d", nt, kw, depth);
 }
 
@@ -116,6 +126,7 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.raw_indices = nullptr;
   a.raw_count = 0;
   a.raw_offset = 0;
+  a.raw_static = 0;
   a.g_delta = a.g_start = a.g_count = a.perm = a.n_groups_dev = nullptr;
   a.n_groups = 0;
   a.uniform_count = 0;
@@ -370,7 +381,15 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
     a.raw_offset = index_offset;
     a.n_groups = prob_n < n_deltas ? prob_n : n_deltas;
     a.accumulate = accumulate;
-    return launch_sparse24(a, pick_nt(prob_n, a.n_groups), 1, static_cast<hipStream_t>(stream));
+    const int nt = pick_nt(prob_n, a.n_groups);
+    // With at least two tokens per delta on average nearly every delta is in use: one group per
+    // delta, whose weights are requested before the indices have arrived (a delta without
+    // tokens costs one prefetched step per wave).  Sparser batches route first.
+    if (prob_n >= 2 * n_deltas && env_int("TRITEIA_HIP_EAGER", 1)) {
+      a.raw_static = 1;
+      a.n_groups = n_deltas;
+    }
+    return launch_sparse24(a, nt, 1, static_cast<hipStream_t>(stream));
   }
   if (int e = triteia_hip_route_plan(token_indices, index_offset, n_deltas, prob_n, workspace, workspace_bytes, dev, stream))
     return e;
