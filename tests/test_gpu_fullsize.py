@@ -41,8 +41,12 @@ def _check_properties(ops, q, me, s, x, idx_np, sample_rows, sample_deltas, what
     for t in sample_rows:
         d = int(idx_np[t])
         if d >= 0:
-            alone = ops.matmul_4bit_2_4(q[d], x[t:t + 1], me[d], s[d])
-            assert torch.equal(alone[0], out[t]), f"{what}: row {t} differs from its own delta's product"
+            # the same row routed on its own (same delta index, hence the same walk over k): same bits
+            alone = ops.sbmm_4bit_2_4_native(q, x[t:t + 1].contiguous(), me, s, idx[t:t + 1].contiguous())
+            assert torch.equal(alone[0], out[t]), f"{what}: row {t} differs from the same row routed on its own"
+            single = ops.matmul_4bit_2_4(q[d], x[t:t + 1], me[d], s[d])
+            err = (single[0].float() - out[t].float()).norm() / single[0].float().norm()
+            assert float(err) < 1e-3, f"{what}: row {t} is {float(err):.2e} from the single-matrix op"
     out2 = ops.sbmm_4bit_2_4_native(q, x * 2, me, s, idx)
     normal = out.abs() >= 2.0 ** -13             # fp16 subnormals round differently after doubling
     assert torch.equal(out2[normal], (out * 2)[normal]), f"{what}: out(2x) != 2 out(x)"

@@ -87,6 +87,7 @@ struct Sparse24Args {
   int n_deltas;             // deltas with index outside [0, n_deltas) are skipped
   int accumulate;           // 0: out = result, 1: out += result
   int raw_static;           // fused routing with group g = delta g: weights are requested before the indices arrive
+  int rot_spread;           // steps between the starting points of consecutive deltas' walks over K (0: n_steps / 16)
   int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run
 #ifdef TRITEIA_HIP_TIMELINE
   long long* timeline;      // [unit][wave][4] 100 MHz timestamps (debug builds only)
@@ -159,6 +160,7 @@ struct TileCtx {
   const _Float16* sc;       // scales of the 128 columns
   long qrow, mrow;          // vectors per packed row (weights, metadata)
   int k_rows, n_steps;      // packed rows, 128-k steps
+  int rot;                  // this delta's walk over K starts at step `rot` and wraps around
   int cb;                   // column block
   int tid, wave, lane, r, q;
   int raw_list;             // fused routing: lane s holds the token row of slot s of the group
@@ -170,17 +172,25 @@ struct TileCtx {
 
 // One pass over K for up to 16*NTT tokens of one group: loads, sparse MFMAs, cross-wave
 // reduction, scaled fp16 store.  `first` = index of the pass's first token in the group's list.
-// USE_PRE: the weights of this wave's first step are already on their way in `pre`.
-template <int NTT, int KW, int DEPTH, bool USE_PRE = false>
+// NPRE: the weights of this wave's first NPRE (<= DEPTH) steps are already on their way in `pre`.
+template <int NTT, int KW, int DEPTH, int NPRE = 0>
 __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int first, int cnt,
                                           float (*red)[16][kRedStride], int* s_rows, const WPre* pre = nullptr) {
   const int r = c.r, q = c.q, wave = c.wave;
   const int k_rows = c.k_rows, n_steps = c.n_steps;
+  // The i-th step of a delta's walk over K is step (i + rot) mod n_steps of the matrix: deltas
+  // that are streamed side by side sit a power of two apart in memory, and in lockstep they
+  // would hit the same DRAM banks at the same moment (measured: 16 deltas of 4096 x 4096
+  // stream at 4.8 TB/s in lockstep, at 5.7 TB/s with their walks spread around the ring).
+  auto phys = [&](int st) {
+    const int ps = st + c.rot;
+    return st < n_steps ? (ps < n_steps ? ps : ps - n_steps) : 0;
+  };
 
   // Steps past the end of K (st >= n_steps) read step 0 again: cheap cache hits that keep the
   // load count per iteration constant; they are never multiplied.
   auto load_w = [&](StepFrag<NTT>& f, int st) {
-    const int tr0 = (st < n_steps ? st : 0) << 2;
+    const int tr0 = phys(st) << 2;
     const int tr = min(tr0 + q, k_rows - 1);  // clamped: rows past the end are cancelled by zero B
     const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
     const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
@@ -203,11 +213,11 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   StepFrag<NTT> ring[DEPTH];
 #pragma unroll
   for (int j = 0; j < DEPTH; j++) {
-    if (USE_PRE && j == 0) {
+    if (j < NPRE) {
 #pragma unroll
-      for (int a = 0; a < 4; a++) ring[0].wq[a] = pre->wq[a];
-      ring[0].mt[0] = pre->mt[0];
-      ring[0].mt[1] = pre->mt[1];
+      for (int a = 0; a < 4; a++) ring[j].wq[a] = pre[j].wq[a];
+      ring[j].mt[0] = pre[j].mt[0];
+      ring[j].mt[1] = pre[j].mt[1];
     } else {
       load_w(ring[j], wave + j * KW);
     }
@@ -235,7 +245,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
     for (int nt = 0; nt < NTT; nt++) acc[cc][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   auto load_x = [&](StepFrag<NTT>& f, int st) {
-    const int tr0 = (st < n_steps ? st : 0) << 2;
+    const int tr0 = phys(st) << 2;
     // rows tr0+2.. may lie past the end of K in the last step: clamp the address, zero at use
     const long xoff_a = (long)min(tr0, k_rows - 1 - (q >> 1)) * 32;
     const long xoff_b = (long)min(tr0 + 2, k_rows - 1 - (q >> 1)) * 32;
@@ -249,7 +259,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   };
 
   auto compute_step = [&](const StepFrag<NTT>& f, int st) {
-    const int tr0 = st << 2;
+    const int tr0 = phys(st) << 2;
     const bool tail = tr0 + 4 > k_rows;            // wave-uniform: only the last, partial step
     const bool ok_a = (tr0 + (q >> 1)) < k_rows;
     const bool ok_b = (tr0 + 2 + (q >> 1)) < k_rows;
@@ -363,7 +373,10 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 // EAGER: fused routing with group g = delta g (Sparse24Args::raw_static): the weights of the first
 // step are requested at once, together with the indices, instead of one memory round trip later.
 template <int NT, int KW, int DEPTH, bool EAGER = false>
-__global__ __launch_bounds__(64 * KW, (NT == 1 ? 3 : (NT == 2 ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
+__global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2 ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
+  // steps per wave requested ahead of the routing in the EAGER build (the 32- and 64-token builds
+  // also hold narrower passes with a ring of their own depth: one step fits them all)
+  constexpr int NPRE = EAGER ? (NT == 1 ? DEPTH : 1) : 0;
   __shared__ float red[KW][16][kRedStride];
   __shared__ int s_rows[16 * NT];
 
@@ -399,12 +412,16 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? 3 : (NT == 2 ? 2 : 1))) void sp
     c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.r >> 3)) * 16 + (c.r & 7);
     c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;
     c.sv = *reinterpret_cast<const half8_t*>(c.sc + (c.tid & 15) * 8);
+    // spread up to 16 side-by-side deltas evenly around the ring of steps (by the delta's index, so
+    // that a result does not depend on where the weights happen to lie in memory)
+    const int spread = p.rot_spread > 0 ? p.rot_spread : max(1, c.n_steps >> 4);
+    c.rot = (int)(((long)delta * spread) % c.n_steps);
   };
 
   // group descriptor and live group count are fetched side by side (no dependent chain);
   // grp < p.n_groups (the host's upper bound) keeps the descriptor reads in bounds
   int delta, start, count;
-  WPre pre;
+  WPre pre[NPRE > 0 ? NPRE : 1];
   if (p.raw_indices) {
     // Fused routing for small batches: every wavefront looks at all (<= 64) indices, one per
     // lane, and works out its delta and the rows routed to it -- a few dozen instructions
@@ -416,13 +433,20 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? 3 : (NT == 2 ? 2 : 1))) void sp
       if (grp >= p.n_deltas) return;
       delta = grp;
       bind_delta(delta);
-      const int tr = min((c.wave << 2) + c.q, c.k_rows - 1);
-      const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
-      const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
 #pragma unroll
-      for (int a = 0; a < 4; a++) pre.wq[a] = wp[a];
-      pre.mt[0] = mp[0];
-      pre.mt[1] = mp[8];
+      for (int j = 0; j < NPRE; j++) {
+        const int st = c.wave + j * KW;              // this wave's j-th step (beyond the end of K: loads go unused)
+        int ps = st + c.rot;
+        if (ps >= c.n_steps) ps -= c.n_steps;
+        if (st >= c.n_steps) ps = 0;
+        const int tr = min((ps << 2) + c.q, c.k_rows - 1);
+        const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
+        const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
+#pragma unroll
+        for (int a = 0; a < 4; a++) pre[j].wq[a] = wp[a];
+        pre[j].mt[0] = mp[0];
+        pre[j].mt[1] = mp[8];
+      }
     }
     d -= p.raw_offset;
     if (c.lane >= p.raw_count || d < 0 || d >= p.n_deltas) d = -1;
@@ -479,11 +503,11 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? 3 : (NT == 2 ? 2 : 1))) void sp
     const int cnt = min(count - t0, 16 * NT);
     if (EAGER && first_pass) {
       if (NT == 1 || cnt <= 16) {
-        tile_pass<1, KW, (NT == 1 ? DEPTH : 2), true>(p, c, start + t0, cnt, red, s_rows, &pre);
+        tile_pass<1, KW, (NT == 1 ? DEPTH : 2), NPRE>(p, c, start + t0, cnt, red, s_rows, pre);
       } else if (NT == 2 || cnt <= 32) {
-        tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), true>(p, c, start + t0, cnt, red, s_rows, &pre);
+        tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), NPRE>(p, c, start + t0, cnt, red, s_rows, pre);
       } else {
-        tile_pass<NT, KW, DEPTH, true>(p, c, start + t0, cnt, red, s_rows, &pre);
+        tile_pass<NT, KW, DEPTH, NPRE>(p, c, start + t0, cnt, red, s_rows, pre);
       }
     } else if (NT == 1 || cnt <= 16) {
       tile_pass<1, KW, (NT == 1 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);

@@ -66,6 +66,7 @@ int pick_nt(long tokens, long groups) {
   if (forced == 1 || forced == 2 || forced == 4) return forced;
   if (groups < 1) groups = 1;
   if (tokens <= 16) return 1;
+  if (tokens <= 6 * groups) return 1;    // typical group well under 16 tokens (a rare larger one takes two passes)
   if (tokens <= 24 * groups) return 2;   // typical group well under 32 tokens
   return 4;
 }
@@ -83,11 +84,13 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   if (tsplit > 65535) tsplit = 65535;
   const long cb_pad = (a.m / 128 + 7) / 8 * 8;   // column blocks padded to the 8 XCDs
   const int kw = env_int("TRITEIA_HIP_KW", 4);
-  // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight, the
-  // 32-token kernel 2 per CU with two, the 64-token kernel 1 per CU with one
-  // (the eager form of fused routing holds one more step of weights: one step in flight for every tile)
-  const int depth = env_int("TRITEIA_HIP_DEPTH", nt == 2 && !(a.raw_indices && a.raw_static) ? 2 : 1);
-  if (a.raw_indices && a.raw_static && !(kw == 4 && depth == 1)) {
+  // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight (2 with
+  // two), the 32-token kernel 2 per CU with two, the 64-token kernel 1 per CU with one.  Fused
+  // routing in its eager form keeps one step in flight (measured: a second step requested ahead of
+  // the routing makes the 16-delta case slower, 23.1 against 22.0 us).
+  const bool eager = a.raw_indices && a.raw_static;
+  const int depth = env_int("TRITEIA_HIP_DEPTH", eager ? 1 : (nt == 2 ? 2 : 1));
+  if (eager && !(kw == 4 && ((nt == 1 && depth == 2) || (nt == 1 && depth == 1) || (nt == 2 && depth == 1) || (nt == 4 && depth == 1)))) {
     a.raw_static = 0;   // no eager build of this variant: route first, then request
     a.n_groups = a.raw_count < a.n_deltas ? a.raw_count : a.n_deltas;
   }
@@ -97,9 +100,9 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
 #define TRY(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
 #define TRY_EAGER(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_, true>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
   if (a.raw_indices && a.raw_static) {
-    TRY_EAGER(1, 4, 1) TRY_EAGER(2, 4, 1) TRY_EAGER(4, 4, 1)
+    TRY_EAGER(1, 4, 1) TRY_EAGER(1, 4, 2) TRY_EAGER(2, 4, 1) TRY_EAGER(4, 4, 1)
   }
-  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 2) TRY(1, 16, 1)
+  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 2)
   TRY(2, 4, 1) TRY(2, 4, 2) TRY(2, 8, 1)
   TRY(4, 4, 1)
 #undef TRY
@@ -135,6 +138,7 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.delta_step = 0;
   a.accumulate = 0;
   a.xcd_swizzle = env_int("TRITEIA_HIP_XCD_SWIZZLE", 1);
+  a.rot_spread = env_int("TRITEIA_HIP_ROT_SPREAD", 0);
 #ifdef TRITEIA_HIP_TIMELINE
   a.timeline = reinterpret_cast<long long*>(strtoull(getenv("TRITEIA_HIP_TIMELINE_PTR") ? getenv("TRITEIA_HIP_TIMELINE_PTR") : "0", nullptr, 0));
 #endif
