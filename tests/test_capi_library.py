@@ -61,7 +61,7 @@ def test_other_argument_errors():
     need = lib.triteia_hip_sbmm_routed_workspace_bytes(64, 16)
     assert need == 4 * (8 + 4 * (16 + 64 // 16) + 4 * (64 // 33 + 1) + 64)
     assert lib.triteia_hip_plan_tile_tokens(8, 8) == 16
-    assert lib.triteia_hip_plan_tile_tokens(64, 16) == 16       # under 6 tokens per delta on average
+    assert lib.triteia_hip_plan_tile_tokens(64, 16) == 16       # at most 4 tokens per delta on average
     assert lib.triteia_hip_plan_tile_tokens(256, 16) == 32
     assert lib.triteia_hip_plan_tile_tokens(4096, 4) == 64
     one = ctypes.c_void_p(16)

@@ -87,7 +87,7 @@ struct Sparse24Args {
   int n_deltas;             // deltas with index outside [0, n_deltas) are skipped
   int accumulate;           // 0: out = result, 1: out += result
   int raw_static;           // fused routing with group g = delta g: weights are requested before the indices arrive
-  int rot_spread;           // steps between the starting points of consecutive deltas' walks over K (0: n_steps / 16)
+  int rot_spread;           // steps between the starting points of consecutive deltas' walks over K (0: all start at step 0)
   int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run
 #ifdef TRITEIA_HIP_TIMELINE
   long long* timeline;      // [unit][wave][4] 100 MHz timestamps (debug builds only)
@@ -412,10 +412,9 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
     c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.r >> 3)) * 16 + (c.r & 7);
     c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;
     c.sv = *reinterpret_cast<const half8_t*>(c.sc + (c.tid & 15) * 8);
-    // spread up to 16 side-by-side deltas evenly around the ring of steps (by the delta's index, so
-    // that a result does not depend on where the weights happen to lie in memory)
-    const int spread = p.rot_spread > 0 ? p.rot_spread : max(1, c.n_steps >> 4);
-    c.rot = (int)(((long)delta * spread) % c.n_steps);
+    // side-by-side deltas start their walks spread around the ring of steps (by the delta's index,
+    // so that a result does not depend on where the weights happen to lie in memory)
+    c.rot = (int)(((long)delta * p.rot_spread) % c.n_steps);
   };
 
   // group descriptor and live group count are fetched side by side (no dependent chain);

@@ -66,7 +66,9 @@ int pick_nt(long tokens, long groups) {
   if (forced == 1 || forced == 2 || forced == 4) return forced;
   if (groups < 1) groups = 1;
   if (tokens <= 16) return 1;
-  if (tokens <= 6 * groups) return 1;    // typical group well under 16 tokens (a rare larger one takes two passes)
+  // small batches spread thinly: groups well under 16 tokens (a rare larger one takes a second pass);
+  // with more tokens some delta of a skewed batch is always hot and 32-token tiles win
+  if (tokens <= 64 && tokens <= 4 * groups) return 1;
   if (tokens <= 24 * groups) return 2;   // typical group well under 32 tokens
   return 4;
 }
@@ -93,6 +95,15 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   if (eager && !(kw == 4 && ((nt == 1 && depth == 2) || (nt == 1 && depth == 1) || (nt == 2 && depth == 1) || (nt == 4 && depth == 1)))) {
     a.raw_static = 0;   // no eager build of this variant: route first, then request
     a.n_groups = a.raw_count < a.n_deltas ? a.raw_count : a.n_deltas;
+  }
+  // About 512 workgroups run at a time.  When those belong to four or more deltas (narrow matrices),
+  // the deltas start their walks over K spread evenly around the ring of steps; wide matrices are
+  // streamed one or two at a time anyway and walk from step 0.
+  {
+    const long side_by_side = 512 / cb_pad;
+    const int n_steps = (a.k / 32 + 3) / 4;
+    const long spread = side_by_side >= 4 ? n_steps / (side_by_side < 16 ? side_by_side : 16) : 0;
+    a.rot_spread = env_int("TRITEIA_HIP_ROT_SPREAD", (int)spread);
   }
   const long units = (long)a.n_groups * cb_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
@@ -138,7 +149,7 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.delta_step = 0;
   a.accumulate = 0;
   a.xcd_swizzle = env_int("TRITEIA_HIP_XCD_SWIZZLE", 1);
-  a.rot_spread = env_int("TRITEIA_HIP_ROT_SPREAD", 0);
+  a.rot_spread = 0;
 #ifdef TRITEIA_HIP_TIMELINE
   a.timeline = reinterpret_cast<long long*>(strtoull(getenv("TRITEIA_HIP_TIMELINE_PTR") ? getenv("TRITEIA_HIP_TIMELINE_PTR") : "0", nullptr, 0));
 #endif
