@@ -91,7 +91,11 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   // routing in its eager form keeps one step in flight (measured: a second step requested ahead of
   // the routing makes the 16-delta case slower, 23.1 against 22.0 us).
   const bool eager = a.raw_indices && a.raw_static;
-  const int depth = env_int("TRITEIA_HIP_DEPTH", eager ? 1 : (nt == 2 ? 2 : 1));
+  // launches that do not fill the GPU twice over (at most 512 workgroups) are bound by the latency
+  // of each wave's chain of requests rather than by bandwidth: a second step in flight pays there
+  // (5-12 % measured) while it costs time on full launches
+  const bool small = (long)a.n_groups * cb_pad * tsplit <= 512;
+  const int depth = env_int("TRITEIA_HIP_DEPTH", eager ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1));
   if (eager && !(kw == 4 && ((nt == 1 && depth == 2) || (nt == 1 && depth == 1) || (nt == 2 && depth == 1) || (nt == 4 && depth == 1)))) {
     a.raw_static = 0;   // no eager build of this variant: route first, then request
     a.n_groups = a.raw_count < a.n_deltas ? a.raw_count : a.n_deltas;
