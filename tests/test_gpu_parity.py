@@ -385,6 +385,8 @@ def _assert_allclose_scaled(got, ref, what):
     (10, 5, 768, 256, 64, 61),        # tests/ops/test_lora_bgmv.py:73
     (128, 2, 4096, 12288, 64, 62),    # tests/ops/test_lora_bgmv.py:74
     (33, 4, 512, 1024, 8, 63), (33, 4, 512, 1024, 16, 64), (33, 4, 512, 1000, 32, 65),
+    # segments longer than one pass of the row slots, ragged tails, a rank that is no power of two, the widest rank
+    (301, 3, 1024, 2048, 16, 66), (71, 3, 512, 520, 24, 67), (41, 2, 1024, 512, 128, 68),
 ])
 def test_lora_ops(ops, T, M, k, m, r, seed):
     say(f"lora T={T} M={M} k={k} m={m} r={r} seed={seed}")

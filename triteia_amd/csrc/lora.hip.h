@@ -14,9 +14,14 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#ifndef TRITEIA_SHRINK_UNROLL
+#define TRITEIA_SHRINK_UNROLL 8
+#endif
+
 namespace triteia_hip {
 
 typedef _Float16 lhalf8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 lhalf2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kLoraMaxNarrow = 128;
 
@@ -98,7 +103,8 @@ struct SgmvArgs {
   const int* perm;
   const int* n_groups_dev;
   const int* n_groups2_dev;
-  int n_groups;
+  int n_groups;               // blocks along x: segments, or the maximum lengths of both tile lists together
+  int max_groups2;            // maximum length of the second tile list
   int n_adapters;
   float scale;
 };
@@ -109,16 +115,19 @@ struct SgmvGroup {
 };
 
 __device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* out) {
-  const int n = a.n_groups_dev ? *a.n_groups_dev : a.n_groups;
-  const int n2 = a.n_groups2_dev ? *a.n_groups2_dev : 0;
-  if (g >= n + n2) return false;
-  int adapter;
+  int adapter, n = a.n_groups, n2 = 0;
   if (a.seg) {
     adapter = g;
     out->start = a.seg[g];
-    out->count = a.seg[g + 1] - a.seg[g];
+    out->count = a.seg[g + 1] - out->start;
   } else {
-    const int4 d = g < n ? a.tiles[g] : a.tiles2[g - n];
+    // the tile is read together with the tile counts (the lists are allocated at their maximum
+    // length, g is inside them); whether it is a live one is decided afterwards
+    const int first = a.n_groups - (a.tiles2 ? a.max_groups2 : 0);   // length of the first list
+    const int4 d = g < first ? a.tiles[g] : a.tiles2[g - first];
+    n = *a.n_groups_dev;
+    n2 = a.n_groups2_dev ? *a.n_groups2_dev : 0;
+    if (g < first ? g >= n : g - first >= n2) return false;
     adapter = d.x;
     out->start = d.y;
     out->count = d.z;
@@ -131,52 +140,80 @@ __device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* 
 
 __device__ __forceinline__ int sgmv_row(const SgmvArgs& a, int i) { return a.perm ? a.perm[i] : i; }
 
-// wide -> narrow (d_out <= DOUT <= 128): grid (n_groups, row slots), block 256; a block computes
-// one token row at a time.  Thread j takes the 8-row slabs j, j + 256, ... of the adapter matrix
-// (8 * d_out consecutive halfs, so a wavefront reads 64 slabs back to back) against 8 activations,
-// keeping d_out partial sums; the 256 partial vectors are then summed by shuffles and LDS.
-template <int DOUT>
+// wide -> narrow (d_out <= DOUT <= 128): grid (n_groups, row slots), block 256; a block takes
+// R token rows of its group at a time and walks all of d_in once for them.  With CB = d_out / 8
+// column blocks, thread (kp, cb) = (tid / CB, tid % CB) reads the 16-byte pieces [k][cb*8 .. +8] of
+// the adapter rows k = 2 kp and 2 kp + 1, then 2 (256 / CB) rows further on, and so on, so that a
+// wavefront's loads cover consecutive memory; the matching two activations of a row are one dword.
+// Each thread keeps R x 8 partial sums; they are summed over the threads of a column block in two
+// passes through LDS (row stride 8 R + 1 floats, so neither pass has bank conflicts worth naming).
+template <int DOUT, int R>
 __global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgs a) {
-  __shared__ float part[4][DOUT];
+  constexpr int V = 8 * R;
+  __shared__ float part[256 * (V + 1)];
+  __shared__ float part2[256];
   SgmvGroup g;
   if (!sgmv_group(a, blockIdx.x, &g)) return;
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
   const int dn = a.d_out;
-  for (int rr = blockIdx.y; rr < g.count; rr += gridDim.y) {
-    const int row = sgmv_row(a, g.start + rr);
-    const _Float16* x = a.x + (long)row * a.x_stride;
-    float acc[DOUT];
+  const int CB = dn >> 3;
+  const int KP = 256 / CB;               // k pairs per sweep of the block
+  const int cb = tid % CB, kp = tid / CB;
+  const bool worker = kp < KP;
+  // second pass: thread (v, cb2, part) adds every P-th partial of output v of column block cb2
+  const int P = 256 / (V * CB);
+  const int v2 = tid % V, cb2 = (tid / V) % CB, part_id = tid / (V * CB);
+  for (int r0 = blockIdx.y * R; r0 < g.count; r0 += gridDim.y * R) {
+    int rows[R];
+    const _Float16* xr[R];
 #pragma unroll
-    for (int j = 0; j < DOUT; j++) acc[j] = 0.f;
-    for (int k0 = tid * 8; k0 < a.d_in; k0 += 256 * 8) {
-      const lhalf8_t xv = *reinterpret_cast<const lhalf8_t*>(x + k0);
-      const _Float16* wk = g.w + (long)k0 * dn;
+    for (int r = 0; r < R; r++) {
+      rows[r] = sgmv_row(a, g.start + (r0 + r < g.count ? r0 + r : r0));
+      xr[r] = a.x + (long)rows[r] * a.x_stride;
+    }
+    float acc[R][8];
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const float xe = (float)xv[e];
+    for (int r = 0; r < R; r++)
 #pragma unroll
-        for (int j0 = 0; j0 < DOUT; j0 += 8) {
-          if (j0 < dn) {
-            const lhalf8_t wv = *reinterpret_cast<const lhalf8_t*>(wk + (long)e * dn + j0);
+      for (int j = 0; j < 8; j++) acc[r][j] = 0.f;
+    if (worker) {
+      const _Float16* wp = g.w + cb * 8;
+#pragma unroll TRITEIA_SHRINK_UNROLL
+      for (int k = 2 * kp; k < a.d_in; k += 2 * KP) {
+        const lhalf8_t w0 = *reinterpret_cast<const lhalf8_t*>(wp + (long)k * dn);
+        const lhalf8_t w1 = *reinterpret_cast<const lhalf8_t*>(wp + (long)(k + 1) * dn);
 #pragma unroll
-            for (int j = 0; j < 8; j++) acc[j0 + j] += xe * (float)wv[j];
-          }
+        for (int r = 0; r < R; r++) {
+          const lhalf2_t xv = *reinterpret_cast<const lhalf2_t*>(xr[r] + k);
+          const float x0 = (float)xv[0], x1 = (float)xv[1];
+#pragma unroll
+          for (int j = 0; j < 8; j++) acc[r][j] += x0 * (float)w0[j] + x1 * (float)w1[j];
         }
       }
     }
 #pragma unroll
-    for (int j = 0; j < DOUT; j++) {
-      const float v = wave_sum(acc[j]);
-      if (lane == 0) part[wave][j] = v;
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) part[tid * (V + 1) + r * 8 + j] = acc[r][j];
+    __syncthreads();
+    if (part_id < P) {
+      float s = 0.f;
+      for (int i = part_id; i < KP; i += P) s += part[(cb2 + CB * i) * (V + 1) + v2];
+      part2[tid] = s;
     }
     __syncthreads();
-    if (tid < dn) {
-      const float sum = part[0][tid] + part[1][tid] + part[2][tid] + part[3][tid];
-      _Float16* yp = a.y + (long)row * a.y_stride + tid;
-      *yp = (_Float16)((float)*yp + sum * a.scale);
+    if (tid < V * CB) {
+      float sum = 0.f;
+      for (int p = 0; p < P; p++) sum += part2[tid + V * CB * p];
+      const int r = v2 >> 3;
+      if (r0 + r < g.count) {
+        int row = rows[0];
+#pragma unroll
+        for (int q = 1; q < R; q++) row = r == q ? rows[q] : row;
+        _Float16* yp = a.y + (long)row * a.y_stride + cb2 * 8 + (v2 & 7);
+        *yp = (_Float16)((float)*yp + sum * a.scale);
+      }
     }
-    __syncthreads();
   }
 }
 
@@ -209,8 +246,9 @@ __global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgs a) {
 
 // narrow -> wide for d_in <= DIN <= 32: grid (n_groups, ceil(d_out / 2048), row slots), block 256.
 // A thread owns 8 consecutive output columns: its d_in x 8 weight patch stays in registers while
-// it walks the group's rows (16-byte loads and stores throughout, no barriers).
-template <int DIN>
+// it walks the group's rows R at a time (16-byte loads and stores throughout, no barriers; the R
+// rows' loads are independent, so they are in flight together).
+template <int DIN, int R>
 __global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgs a) {
   SgmvGroup g;
   if (!sgmv_group(a, blockIdx.x, &g)) return;
@@ -222,28 +260,34 @@ __global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgs a) 
     if (i < a.d_in) w[i] = *reinterpret_cast<const lhalf8_t*>(g.w + (long)i * a.d_out + j0);
     else w[i] = lhalf8_t{0, 0, 0, 0, 0, 0, 0, 0};
   }
-  for (int rr = blockIdx.z; rr < g.count; rr += gridDim.z) {
-    const int row = sgmv_row(a, g.start + rr);
-    const _Float16* xr = a.x + (long)row * a.x_stride;
-    float acc[8];
+  for (int r0 = blockIdx.z * R; r0 < g.count; r0 += gridDim.z * R) {
+    lhalf8_t xv[R][DIN / 8], old[R];
+    _Float16* yp[R];
 #pragma unroll
-    for (int e = 0; e < 8; e++) acc[e] = 0.f;
+    for (int r = 0; r < R; r++) {
+      const int row = sgmv_row(a, g.start + (r0 + r < g.count ? r0 + r : r0));
+      const _Float16* xr = a.x + (long)row * a.x_stride;
+      yp[r] = a.y + (long)row * a.y_stride + j0;
 #pragma unroll
-    for (int i0 = 0; i0 < DIN; i0 += 8) {
-      if (i0 < a.d_in) {
-        const lhalf8_t xv = *reinterpret_cast<const lhalf8_t*>(xr + i0);   // same address in every lane
-#pragma unroll
-        for (int i = 0; i < 8; i++)
-#pragma unroll
-          for (int e = 0; e < 8; e++) acc[e] += (float)xv[i] * (float)w[i0 + i][e];
-      }
+      for (int i0 = 0; i0 < DIN / 8; i0++)
+        xv[r][i0] = i0 * 8 < a.d_in ? *reinterpret_cast<const lhalf8_t*>(xr + i0 * 8)   // same address in every lane
+                                    : lhalf8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      old[r] = *reinterpret_cast<const lhalf8_t*>(yp[r]);
     }
-    _Float16* yp = a.y + (long)row * a.y_stride + j0;
-    const lhalf8_t old = *reinterpret_cast<const lhalf8_t*>(yp);
-    lhalf8_t o;
 #pragma unroll
-    for (int e = 0; e < 8; e++) o[e] = (_Float16)((float)old[e] + acc[e] * a.scale);
-    *reinterpret_cast<lhalf8_t*>(yp) = o;
+    for (int r = 0; r < R; r++) {
+      float acc[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc[e] = 0.f;
+#pragma unroll
+      for (int i = 0; i < DIN; i++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += (float)xv[r][i / 8][i % 8] * (float)w[i][e];
+      lhalf8_t o;
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = (_Float16)((float)old[r][e] + acc[e] * a.scale);
+      if (r == 0 || r0 + r < g.count) *reinterpret_cast<lhalf8_t*>(yp[r]) = o;
+    }
   }
 }
 

@@ -444,6 +444,15 @@ size_t triteia_hip_sgmv_tmp_size(int num_problems) {
   return num_problems > 0 ? (size_t)60 * (size_t)num_problems : 0;
 }
 
+#ifndef TRITEIA_SHRINK_ROWS16
+#define TRITEIA_SHRINK_ROWS16 2
+#endif
+#ifndef TRITEIA_EXPAND_ROWS16
+#define TRITEIA_EXPAND_ROWS16 4
+#endif
+constexpr int kShrinkRows16 = TRITEIA_SHRINK_ROWS16;   // token rows a block of the rank <= 16 shrink kernel takes at a time
+constexpr int kExpandRows16 = TRITEIA_EXPAND_ROWS16;
+
 static int launch_sgmv(SgmvArgs a, int max_rows, hipStream_t st) {
   const int narrow = a.d_in < a.d_out ? a.d_in : a.d_out;
   if (a.d_in % 8 != 0 || a.d_out % 8 != 0 || narrow > kLoraMaxNarrow)
@@ -452,18 +461,18 @@ static int launch_sgmv(SgmvArgs a, int max_rows, hipStream_t st) {
   // rows of a group are spread over y (shrink) / z (expand); group sizes live on the device
   int row_slots = max_rows < 64 ? max_rows : 64;
   if (row_slots < 1) row_slots = 1;
+  auto slots = [&](int rows_per_block) { return (row_slots + rows_per_block - 1) / rows_per_block; };
   if (a.d_in >= a.d_out) {
-    const dim3 grid(a.n_groups, row_slots);
-    if (a.d_out <= 16) hipLaunchKernelGGL((sgmv_shrink_kernel<16>), grid, dim3(256), 0, st, a);
-    else if (a.d_out <= 32) hipLaunchKernelGGL((sgmv_shrink_kernel<32>), grid, dim3(256), 0, st, a);
-    else if (a.d_out <= 64) hipLaunchKernelGGL((sgmv_shrink_kernel<64>), grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((sgmv_shrink_kernel<128>), grid, dim3(256), 0, st, a);
+    if (a.d_out <= 16) hipLaunchKernelGGL((sgmv_shrink_kernel<16, kShrinkRows16>), dim3(a.n_groups, slots(kShrinkRows16)), dim3(256), 0, st, a);
+    else if (a.d_out <= 32) hipLaunchKernelGGL((sgmv_shrink_kernel<32, 2>), dim3(a.n_groups, slots(2)), dim3(256), 0, st, a);
+    else if (a.d_out <= 64) hipLaunchKernelGGL((sgmv_shrink_kernel<64, 1>), dim3(a.n_groups, slots(1)), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((sgmv_shrink_kernel<128, 1>), dim3(a.n_groups, slots(1)), dim3(256), 0, st, a);
   } else {
     const int rz = row_slots < 8 ? row_slots : 8;
     const dim3 grid(a.n_groups, (a.d_out + 255) / 256, rz);
-    const dim3 vgrid(a.n_groups, (a.d_out + 2047) / 2048, row_slots < 32 ? row_slots : 32);
-    if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_vec_kernel<16>), vgrid, dim3(256), 0, st, a);
-    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_vec_kernel<32>), vgrid, dim3(256), 0, st, a);
+    const int col_blocks = (a.d_out + 2047) / 2048;
+    if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_vec_kernel<16, kExpandRows16>), dim3(a.n_groups, col_blocks, slots(kExpandRows16)), dim3(256), 0, st, a);
+    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_vec_kernel<32, 2>), dim3(a.n_groups, col_blocks, slots(2)), dim3(256), 0, st, a);
     else if (a.d_in <= 64) hipLaunchKernelGGL((sgmv_expand_kernel<64>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((sgmv_expand_kernel<128>), grid, dim3(256), 0, st, a);
   }
@@ -526,6 +535,7 @@ int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride
     a.tiles2 = reinterpret_cast<const int4*>(ws + L.wide);
     a.n_groups2_dev = ws + L.header + 4;
     a.n_groups += L.max_wide;
+    a.max_groups2 = L.max_wide;
   }
   a.n_adapters = n_adapters;
   a.scale = scale;
