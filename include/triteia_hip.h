@@ -109,13 +109,19 @@ TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n
 
 /* Only the routing step of the call above: fills `workspace` (16-byte aligned) with
  *   int32 header[8] = {narrow tiles, routed tokens, deltas in use, narrow tile size,
- *                      wide tiles, 0, 0, 0}
+ *                      wide tiles, tiles of all[], 0, 0}
  *   int32 tiles[max_tiles][4] = {delta, start, count, 0}: at most `tile size` tokens of one
  *         delta, listed at perm[start .. start+count); a delta's tiles are adjacent
- *   int32 wide[max_wide][4]   = the same for 64-token tiles; only batches of at least 4096
- *         tokens (environment TRITEIA_HIP_WIDE_MIN_BATCH) get any: a delta with c tokens then has c/64 full wide tiles, one more if
+ *   int32 wide[max_wide][4]   = the same for 64-token tiles; only batches of at least 256
+ *         tokens (environment TRITEIA_HIP_WIDE_MIN_BATCH) with at least 8 tokens per delta on
+ *         average get any: a delta with c tokens then has c/64 full wide tiles, one more if
  *         the rest exceeds 32 tokens, and narrow tiles for a smaller rest
  *   int32 perm[prob_n] = token rows grouped by delta, original order kept (stable)
+ *   int32 all[max_tiles][4]   = at the next multiple of 4 ints: for plans with wide tiles, the
+ *         same tokens cut into narrow tiles only (header[5] of them).  The multiply kernels pick
+ *         {tiles, wide} or {all} per weight shape on the device: the wide kernel runs only if
+ *         its tiles fill the chip (wide tiles x ceil(prob_m / 512) >= 200, environment
+ *         TRITEIA_HIP_PLAN_WIDE_MIN_UNITS); the LoRA path always takes all[].
  * with max_tiles = min(prob_n, n_deltas) + prob_n / 16 and max_wide = prob_n / 33 + 1.  The
  * narrow tile size is triteia_hip_plan_tile_tokens(prob_n, n_deltas).  Exposed so that one
  * routing pass can serve every layer of a forward pass and the LoRA path. */

@@ -59,7 +59,7 @@ def test_other_argument_errors():
     assert lib.triteia_hip_bgmv(null, null, null, null, 4, 4096, 16, 1, 3, 1.0, 0, null) == _ffi.ERR_PROB_SHAPE
     # routed sbmm: workspace too small, too many deltas
     need = lib.triteia_hip_sbmm_routed_workspace_bytes(64, 16)
-    assert need == 4 * (8 + 4 * (16 + 64 // 16) + 4 * (64 // 33 + 1) + 64)
+    assert need == 4 * (8 + 4 * (16 + 64 // 16) + 4 * (64 // 33 + 1) + 64 + 4 * (16 + 64 // 16))
     assert lib.triteia_hip_plan_tile_tokens(8, 8) == 16
     assert lib.triteia_hip_plan_tile_tokens(64, 16) == 16       # at most 4 tokens per delta on average
     assert lib.triteia_hip_plan_tile_tokens(256, 16) == 32

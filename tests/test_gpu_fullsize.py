@@ -38,12 +38,20 @@ def _check_properties(ops, q, me, s, x, idx_np, sample_rows, sample_deltas, what
     out = ops.sbmm_4bit_2_4_native(q, x, me, s, idx)
     torch.cuda.synchronize()
     assert bool((out[idx < 0] == 0).all()), f"{what}: -1 rows must stay zero"
+    # Batches of at least 256 tokens with at least 8 tokens per delta carry 64-token wide tiles for
+    # deltas with more than 32 tokens; the wide kernel sums over k in another order than the narrow
+    # one, so only rows of deltas with at most 32 tokens are comparable bit for bit.
+    T, N = x.shape[0], q.shape[0]
+    counts = np.bincount(idx_np[idx_np >= 0], minlength=N)
+    may_be_wide = counts > 32 if (T >= 256 and T >= 8 * min(T, N)) else np.zeros(N, dtype=bool)
+    exact_rows = torch.from_numpy((idx_np < 0) | ~may_be_wide[np.maximum(idx_np, 0)]).to(DEV)
     for t in sample_rows:
         d = int(idx_np[t])
         if d >= 0:
             # the same row routed on its own (same delta index, hence the same walk over k): same bits
             alone = ops.sbmm_4bit_2_4_native(q, x[t:t + 1].contiguous(), me, s, idx[t:t + 1].contiguous())
-            assert torch.equal(alone[0], out[t]), f"{what}: row {t} differs from the same row routed on its own"
+            if not may_be_wide[d]:
+                assert torch.equal(alone[0], out[t]), f"{what}: row {t} differs from the same row routed on its own"
             single = ops.matmul_4bit_2_4(q[d], x[t:t + 1], me[d], s[d])
             err = (single[0].float() - out[t].float()).norm() / single[0].float().norm()
             assert float(err) < 1e-3, f"{what}: row {t} is {float(err):.2e} from the single-matrix op"
@@ -53,7 +61,8 @@ def _check_properties(ops, q, me, s, x, idx_np, sample_rows, sample_deltas, what
     assert float((out2.float() - 2 * out.float()).abs().max()) <= 2.0 ** -23
     perm = torch.randperm(x.shape[0], generator=torch.Generator().manual_seed(1)).to(DEV)
     outp = ops.sbmm_4bit_2_4_native(q, x[perm].contiguous(), me, s, idx[perm].contiguous())
-    assert torch.equal(outp, out[perm]), f"{what}: token order changes the result"
+    assert torch.equal(outp[exact_rows[perm]], out[perm][exact_rows[perm]]), f"{what}: token order changes the result"
+    assert float((outp.float() - out[perm].float()).norm()) <= 1e-3 * float(out.float().norm())
     for d in sample_deltas:
         rows = torch.nonzero(idx == d).flatten()
         if rows.numel() == 0:

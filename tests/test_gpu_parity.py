@@ -19,12 +19,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-WIDE_MIN_BATCH = 512          # the tests lower the batch size from which plans carry wide tiles
+WIDE_MIN_BATCH = 512          # in these tests plans carry wide tiles from this batch size on ...
 
 
 @pytest.fixture(autouse=True)
 def _wide_tiles_from_512_tokens(monkeypatch):
     monkeypatch.setenv("TRITEIA_HIP_WIDE_MIN_BATCH", str(WIDE_MIN_BATCH))
+    # ... and the wide kernel takes them however few they are (by default only when they fill the chip)
+    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
 
 
 def say(msg):
@@ -250,7 +252,7 @@ def _exact_problem(T, N, k, m, seed):
 
 
 @pytest.mark.parametrize("T,N,k,m,seed", [(64, 16, 512, 384, 51), (37, 5, 1024, 256, 52), (300, 7, 512, 640, 53), (700, 3, 256, 512, 54)])
-def test_routing_is_bit_exact_on_exact_arithmetic(ops, T, N, k, m, seed):
+def test_routing_is_bit_exact_on_exact_arithmetic(ops, monkeypatch, T, N, k, m, seed):
     """With inputs on which floating point is exact, every path (fused routing, routing plan with narrow
     and wide tiles, run table, one launch per run, one matmul per delta) must reproduce the oracle bit
     for bit: any token sent to the wrong delta, any row written twice or not at all would show."""
@@ -262,6 +264,11 @@ def test_routing_is_bit_exact_on_exact_arithmetic(ops, T, N, k, m, seed):
     gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
     want = torch.from_numpy(ref.astype(np.float16)).to(DEV)
     assert torch.equal(ops.sbmm_4bit_2_4_native(gq, gx, gm, gs, gi), want)
+    # a plan with wide tiles also carries a narrow-only cut of the same tokens; the kernels choose on the
+    # device (here: a bar no launch reaches, so the narrow-only cut runs and the wide launch returns at once)
+    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1000000000")
+    assert torch.equal(ops.sbmm_4bit_2_4_native(gq, gx, gm, gs, gi), want)
+    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
     assert torch.equal(ops.sbmm_4bit_2_4_forloop(gq, gx, gm, gs, gi), want)
     order = np.argsort(idx, kind="stable")
     gxs, gis = to_gpu(x[order], idx[order])
@@ -340,10 +347,12 @@ def test_route_plan_is_a_stable_grouping():
         tiles = plan[o_tiles:o_tiles + 4 * max_tiles].reshape(max_tiles, 4)[:n_tiles]
         wides = plan[o_wide:o_wide + 4 * max_wide].reshape(max_wide, 4)[:n_wide]
         perm = plan[o_perm:o_perm + T]
+        o_all = (o_perm + T + 3) // 4 * 4
+        alls = plan[o_all:o_all + 4 * max_tiles].reshape(max_tiles, 4)[:plan[5]]
         used = np.unique(d[valid])
         assert tile_dev == tile and n_used == len(used) and n_routed == valid.sum()
-        has_wide = T >= 512
-        pos, ti, wi = 0, 0, 0
+        has_wide = T >= WIDE_MIN_BATCH and T >= 8 * min(T, N)
+        pos, ti, wi, ai = 0, 0, 0, 0
         for delta in used:
             rows = np.nonzero(d == delta)[0]                # ascending = original order
             c = len(rows)
@@ -359,8 +368,13 @@ def test_route_plan_is_a_stable_grouping():
             for first in range(c_wide, c, tile):             # ... then the narrow rest
                 assert list(tiles[ti]) == [delta, pos + first, min(tile, c - first), 0]
                 ti += 1
+            if has_wide:                                     # and the same tokens in narrow tiles only
+                for first in range(0, c, tile):
+                    assert list(alls[ai]) == [delta, pos + first, min(tile, c - first), 0]
+                    ai += 1
             pos += c
-        assert ti == n_tiles and wi == n_wide
+        assert ti == n_tiles and wi == n_wide and ai == plan[5]
+        assert has_wide == (n_wide > 0 or plan[5] > 0) or not valid.any()
 
 
 # ------------------------------------------------------------- lora / ldmm

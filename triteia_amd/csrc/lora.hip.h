@@ -99,12 +99,9 @@ struct SgmvArgs {
   // routing plan's tile list {adapter, start, count, 0} + perm
   const int* seg;
   const int4* tiles;
-  const int4* tiles2;         // second tile list (the plan's wide tiles), after the first
   const int* perm;
   const int* n_groups_dev;
-  const int* n_groups2_dev;
-  int n_groups;               // blocks along x: segments, or the maximum lengths of both tile lists together
-  int max_groups2;            // maximum length of the second tile list
+  int n_groups;               // blocks along x: segments, or the maximum length of the tile list
   int n_adapters;
   float scale;
 };
@@ -115,19 +112,17 @@ struct SgmvGroup {
 };
 
 __device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* out) {
-  int adapter, n = a.n_groups, n2 = 0;
+  int adapter, n = a.n_groups;
   if (a.seg) {
     adapter = g;
     out->start = a.seg[g];
     out->count = a.seg[g + 1] - out->start;
   } else {
-    // the tile is read together with the tile counts (the lists are allocated at their maximum
-    // length, g is inside them); whether it is a live one is decided afterwards
-    const int first = a.n_groups - (a.tiles2 ? a.max_groups2 : 0);   // length of the first list
-    const int4 d = g < first ? a.tiles[g] : a.tiles2[g - first];
+    // the tile is read together with the tile count (the list is allocated at its maximum
+    // length, g is inside it); whether it is a live one is decided afterwards
+    const int4 d = a.tiles[g];
     n = *a.n_groups_dev;
-    n2 = a.n_groups2_dev ? *a.n_groups2_dev : 0;
-    if (g < first ? g >= n : g - first >= n2) return false;
+    if (g >= n) return false;
     adapter = d.x;
     out->start = d.y;
     out->count = d.z;

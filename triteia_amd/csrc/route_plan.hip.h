@@ -9,15 +9,17 @@
 // Output (all int32, in the caller's workspace):
 //   header[0] = number of narrow tiles, header[1] = number of routed tokens,
 //   header[2] = number of deltas that have at least one token, header[3] = narrow tile size,
-//   header[4] = number of wide tiles, header[5..7] = 0
+//   header[4] = number of wide tiles, header[5] = number of tiles in all[], header[6..7] = 0
 //   tiles[..] = {delta, start, count, 0}: `count` <= tile size tokens of one delta,
 //               listed at perm[start .. start+count); ascending delta id, a delta's
 //               tiles are adjacent
 //   wide[..]  = same, for 64-token tiles (only when built with wide = 1): a delta with c
 //               tokens gets c/64 full wide tiles, one more if the rest exceeds 32 tokens,
-//               and narrow tiles for a smaller rest
+//               and narrow tiles (in tiles[]) for a smaller rest
 //   perm[routed] = token rows, grouped by delta, original order kept inside a
 //               delta (stable)
+//   all[..]   = (only with wide = 1) the same tokens cut into narrow tiles only: the consumer
+//               chooses between {tiles, wide} and {all} per weight shape, on the device
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -33,7 +35,7 @@ constexpr int kPlanCachedTokens = 8192;  // token indices kept in LDS between th
 constexpr int kPlanMinTile = 16;      // smallest tile size a plan can be built for
 
 struct PlanLayout {
-  int header, tiles, wide, perm, total;  // offsets in ints
+  int header, tiles, wide, perm, all, total;  // offsets in ints
   int max_tiles, max_wide;
 };
 
@@ -48,7 +50,8 @@ __host__ __device__ inline PlanLayout plan_layout(int n_tokens, int n_deltas) {
   l.tiles = kPlanHeaderInts;
   l.wide = l.tiles + 4 * l.max_tiles;
   l.perm = l.wide + 4 * l.max_wide;
-  l.total = l.perm + n_tokens;
+  l.all = (l.perm + n_tokens + 3) & ~3;
+  l.total = l.all + 4 * l.max_tiles;
   return l;
 }
 
@@ -91,13 +94,14 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
   if (tid < 64) {
     // exclusive scans over the deltas, 64 per iteration: token counts -> first slot in perm,
     // tile counts -> first tile
-    int running = 0, tiles = 0, wides = 0, groups = 0;
+    int running = 0, tiles = 0, wides = 0, alls = 0, groups = 0;
     int4* tile_out = reinterpret_cast<int4*>(ws + L.tiles);
     int4* wide_out = reinterpret_cast<int4*>(ws + L.wide);
+    int4* all_out = reinterpret_cast<int4*>(ws + L.all);
     for (int base = 0; base < n_deltas; base += 64) {
       const int d = base + lane;
       const int c = d < n_deltas ? s_cursor[d] : 0;
-      int chunk_tokens, chunk_tiles, chunk_wides;
+      int chunk_tokens, chunk_tiles, chunk_wides, chunk_alls;
       const int offs = running + wave_excl_scan(c, lane, &chunk_tokens);
       // split this delta's tokens: wide tiles first, the rest in narrow tiles
       int nw = 0, c_wide = 0;
@@ -118,6 +122,15 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
         const int first = i * tile;
         tile_out[tpos + i] = make_int4(d, offs + c_wide + first, min(tile, c_rest - first), 0);
       }
+      if (wide) {
+        const int na = (c + tile - 1) / tile;
+        const int apos = alls + wave_excl_scan(na, lane, &chunk_alls);
+        for (int i = 0; i < na; i++) {
+          const int first = i * tile;
+          all_out[apos + i] = make_int4(d, offs + first, min(tile, c - first), 0);
+        }
+        alls += chunk_alls;
+      }
       if (d < n_deltas) s_cursor[d] = offs;
       running += chunk_tokens;
       tiles += chunk_tiles;
@@ -130,7 +143,7 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
       ws[L.header + 2] = groups;
       ws[L.header + 3] = tile;
       ws[L.header + 4] = wides;
-      ws[L.header + 5] = 0;
+      ws[L.header + 5] = alls;
       ws[L.header + 6] = 0;
       ws[L.header + 7] = 0;
     }

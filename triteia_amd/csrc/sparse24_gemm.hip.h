@@ -79,6 +79,16 @@ struct Sparse24Args {
   const int* g_count;
   const int* perm;          // row of the i-th listed token (nullptr: identity)
   const int* n_groups_dev;  // device-side group count (nullptr: n_groups)
+  // A routing plan with wide tiles lists its tokens twice: as {wide tiles + narrow rest} and as
+  // narrow tiles only.  Which of the two runs is decided on the device, where the number of wide
+  // tiles is known: the wide kernel only pays when its launch fills the chip, i.e. when
+  // wide tiles x wide_gate (column groups per tile) >= wide_min_units.  For the narrow kernel
+  // tiles_alt is the narrow-only list and n_groups_dev points at the plan header ([0] narrow rest
+  // tiles, [4] wide tiles, [5] tiles of the narrow-only list); for the wide kernels n_groups_dev
+  // points at header[4] and wide_min_units != 0 switches the check on.
+  const int4* tiles_alt;
+  int wide_gate;
+  int wide_min_units;
   int n_groups;             // upper bound on the number of groups
   int uniform_count;
   int uniform_stride;
@@ -420,6 +430,7 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   // group descriptor and live group count are fetched side by side (no dependent chain);
   // grp < p.n_groups (the host's upper bound) keeps the descriptor reads in bounds
   int delta, start, count;
+  bool alt_list = false;
   WPre pre[NPRE > 0 ? NPRE : 1];
   if (p.raw_indices) {
     // Fused routing for small batches: every wavefront looks at all (<= 64) indices, one per
@@ -476,7 +487,15 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
       return;
     }
   } else if (p.tiles) {
-    const int4 d = p.tiles[grp];
+    int4 d = p.tiles[grp];
+    if (p.tiles_alt) {
+      // both candidates and the header are requested together; the choice costs no extra round trip
+      const int4 d_alt = p.tiles_alt[grp];
+      if ((long)p.n_groups_dev[4] * p.wide_gate < p.wide_min_units) {
+        d = d_alt;
+        alt_list = true;
+      }
+    }
     delta = d.x;
     start = d.y;
     count = d.z;
@@ -490,7 +509,7 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
     count = p.uniform_count;
   }
   if (!EAGER) {
-    const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
+    const int n_groups = p.n_groups_dev ? p.n_groups_dev[alt_list ? 5 : 0] : p.n_groups;
     if (grp >= n_groups) return;
     if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
     bind_delta(delta);

@@ -62,6 +62,7 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
     count = min(kWideTokens, p.uniform_count - tc * kWideTokens);
   }
   const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
+  if (p.wide_min_units && (long)n_groups * p.wide_gate < p.wide_min_units) return;   // the narrow kernel has taken these tokens
   if (grp >= n_groups) return;
   if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
   const int cnt = min(count, kWideTokens);

@@ -67,6 +67,7 @@ __global__ __launch_bounds__(256, 1) void sparse24_wide128_kernel(const Sparse24
     count = min(kWide128Tokens, p.uniform_count - tc * kWide128Tokens);
   }
   const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
+  if (p.wide_min_units && (long)n_groups * p.wide_gate < p.wide_min_units) return;   // the narrow kernel has taken these tokens
   if (grp >= n_groups) return;
   if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
   const int cnt = min(count, kWide128Tokens);

@@ -127,6 +127,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
 
 void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
                   int prob_k, int n_deltas) {
+  a = Sparse24Args{};   // every field the caller does not set is zero / null
   a.x = static_cast<const _Float16*>(A);
   a.x_stride = prob_k;
   a.qweight = static_cast<const uint4_t*>(B);
@@ -321,12 +322,16 @@ int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas) {
   return 16 * pick_nt(prob_n, prob_n < n_deltas ? prob_n : n_deltas);
 }
 
-// A plan carries wide (64-token) tiles only for batches large enough that whole deltas become
-// bound by the matrix cores (the plan is independent of the layer shape, so the rule only looks
-// at the batch).  Below that, re-reading a hot delta's weights from cache in 32-token tiles is
-// cheaper than a second, poorly filled launch.
-static int plan_has_wide(int prob_n) {
-  return wide_enabled() && prob_n >= env_int("TRITEIA_HIP_WIDE_MIN_BATCH", 4096);
+// A plan carries wide (64-token) tiles, next to a narrow-only cut of the same tokens, for batches
+// with at least 8 tokens per delta on average (the plan is independent of the layer shape, so the
+// rule only looks at the batch).  Which of the two cuts a layer uses is decided on the device:
+// the wide kernel takes its tiles only if they fill the chip (wide tiles x column groups of the
+// layer >= kPlanWideMinUnits); otherwise re-reading a hot delta's weights from cache in narrow
+// tiles is cheaper than a second, poorly filled launch, and the wide launch returns at once.
+constexpr int kPlanWideMinUnits = 200;
+static int plan_has_wide(int prob_n, int n_deltas) {
+  const long groups = n_deltas < prob_n ? n_deltas : prob_n;
+  return wide_enabled() && prob_n >= env_int("TRITEIA_HIP_WIDE_MIN_BATCH", 256) && prob_n >= 8 * groups;
 }
 
 int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
@@ -344,7 +349,7 @@ int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_de
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   hipLaunchKernelGGL(route_plan_kernel, dim3(1), dim3(kPlanThreads), 0, static_cast<hipStream_t>(stream),
                      static_cast<const int*>(token_indices), prob_n, n_deltas, index_offset,
-                     triteia_hip_plan_tile_tokens(prob_n, n_deltas), plan_has_wide(prob_n), static_cast<int*>(workspace));
+                     triteia_hip_plan_tile_tokens(prob_n, n_deltas), plan_has_wide(prob_n, n_deltas), static_cast<int*>(workspace));
   return check_launch("route_plan_kernel");
 }
 
@@ -368,14 +373,25 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
   a.n_groups_dev = ws + L.header;
   a.n_groups = plan_max_tiles(prob_n, n_deltas, tile);
   a.accumulate = accumulate;
+  const bool wide = plan_has_wide(prob_n, n_deltas);
+  bool wide_launch = false;
+  if (wide) {
+    a.tiles_alt = reinterpret_cast<const int4*>(ws + L.all);
+    a.wide_gate = (prob_m / 128 + 3) / 4;
+    a.wide_min_units = env_int("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", kPlanWideMinUnits);
+    // The wide kernel needs whole 128-deep K steps, and a batch that could not reach the bar
+    // even with most of its tokens in wide tiles (one per 48 tokens) is not worth the empty
+    // launch: then the bar is out of reach on the device too and every tile list is the narrow-only one.
+    wide_launch = prob_k % 128 == 0 && (long)(prob_n / 48 + 1) * a.wide_gate >= a.wide_min_units;
+    if (!wide_launch) a.wide_min_units = 0x7fffffff;
+  }
   if (int e = launch_sparse24(a, tile / 16, 1, static_cast<hipStream_t>(stream))) return e;
-  if (plan_has_wide(prob_n)) {
+  if (wide_launch) {
     a.tiles = reinterpret_cast<const int4*>(ws + L.wide);
+    a.tiles_alt = nullptr;
     a.n_groups_dev = ws + L.header + 4;
     a.n_groups = L.max_wide;
-    if (prob_k % 128 == 0) return launch_wide(a, static_cast<hipStream_t>(stream));
-    // a partial last K step needs the narrow kernel: it walks the 64-token tiles in 16*nt-token passes
-    return launch_sparse24(a, tile / 16, (kWideTokens + tile - 1) / tile, static_cast<hipStream_t>(stream));
+    return launch_wide(a, static_cast<hipStream_t>(stream));
   }
   return TRITEIA_HIP_OK;
 }
@@ -527,16 +543,12 @@ int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride
   a.d_out = d_out;
   a.w_base = static_cast<const _Float16*>(w_base);
   a.w_stride = w_stride;
-  a.tiles = reinterpret_cast<const int4*>(ws + L.tiles);
+  // a plan with wide tiles also lists all its tokens in narrow tiles: that is the cut for LoRA
+  const bool wide = plan_has_wide(prob_n, n_adapters);
+  a.tiles = reinterpret_cast<const int4*>(ws + (wide ? L.all : L.tiles));
   a.perm = ws + L.perm;
-  a.n_groups_dev = ws + L.header;
+  a.n_groups_dev = ws + L.header + (wide ? 5 : 0);
   a.n_groups = plan_max_tiles(prob_n, n_adapters, triteia_hip_plan_tile_tokens(prob_n, n_adapters));
-  if (plan_has_wide(prob_n)) {
-    a.tiles2 = reinterpret_cast<const int4*>(ws + L.wide);
-    a.n_groups2_dev = ws + L.header + 4;
-    a.n_groups += L.max_wide;
-    a.max_groups2 = L.max_wide;
-  }
   a.n_adapters = n_adapters;
   a.scale = scale;
   return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream));
