@@ -457,6 +457,8 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
         pre[j].mt[0] = mp[0];
         pre[j].mt[1] = mp[8];
       }
+      // nothing that needs the indices may be scheduled (with its wait) ahead of these requests
+      __builtin_amdgcn_sched_barrier(0);
     }
     d -= p.raw_offset;
     if (c.lane >= p.raw_count || d < 0 || d >= p.n_deltas) d = -1;
