@@ -5,7 +5,7 @@ delta indices[t] - M; -1 means base model only.
 """
 import torch
 
-from triteia_amd.python.capi import add_lora_bgmv, sbmm_2_4_routed
+from triteia_amd.python.capi import route_plan, sbmm_2_4_routed, sgmv_routed
 from .lora import lora_forloop
 from .sbmm import sbmm_4bit_2_4_forloop
 
@@ -31,8 +31,11 @@ def baseline_ldmm(indices, x, LwA, LwB, DeltaW, metas, ss, base_weight=None, deb
 
 
 def ldmm(indices, x, LwA, LwB, DeltaW, metas, ss, base_weight=None, debug=False):
-    """One BGMV pass for the LoRA tokens plus one routed sparse pass for the delta tokens, both
-    accumulating in place into the base output; no gathers, no host synchronisation.
+    """One routed LoRA pass (shrink + expand) for the LoRA tokens plus one routed sparse pass for
+    the delta tokens, both accumulating in place into the base output; no gathers, no host
+    synchronisation.  The reference routes the LoRA tokens through BGMV, which wants every
+    adapter transposed on each call (ldmm.py:93-105); the routed SGMV kernels
+    read LwA / LwB as they are, one routing pass serving both of its stages.
 
     indices int [B]; x [B, H1]; LwA [M, H1, R]; LwB [M, R, H2]; DeltaW / metas / ss the stacked
     packed deltas.  Returns [B, H2] in x.dtype."""
@@ -43,12 +46,13 @@ def ldmm(indices, x, LwA, LwB, DeltaW, metas, ss, base_weight=None, debug=False)
     else:
         y = torch.zeros(x_.shape[0], LwB.shape[2], dtype=x_.dtype, device=x_.device)
     M = LwA.shape[0]
+    idx32 = indices.to(torch.int32)
     if M > 0:
-        # adapters >= M are not LoRA tokens: map them to -1 for the BGMV kernels
-        lora_idx = torch.where(indices < M, indices, -1).to(torch.long)
-        LwA_T = LwA.to(torch.float16).transpose(1, 2).contiguous().unsqueeze(1)
-        LwB_T = LwB.to(torch.float16).transpose(1, 2).contiguous().unsqueeze(1)
-        add_lora_bgmv(y, x_, LwA_T, LwB_T, lora_idx, layer_idx=0, scale=1.0)
+        # the plan over M adapters skips -1 and every index >= M (the delta tokens)
+        plan = route_plan(idx32, M)
+        v = torch.zeros((x_.shape[0], LwA.shape[2]), dtype=torch.float16, device=x_.device)
+        sgmv_routed(v, x_, LwA.to(torch.float16).contiguous(), plan)
+        sgmv_routed(y, v, LwB.to(torch.float16).contiguous(), plan)
     if DeltaW.shape[0] > 0:
-        sbmm_2_4_routed(x_, DeltaW, metas, y, ss, indices.to(torch.int32), index_offset=M, accumulate=True)
+        sbmm_2_4_routed(x_, DeltaW, metas, y, ss, idx32, index_offset=M, accumulate=True)
     return y.to(x.dtype)
