@@ -313,6 +313,43 @@ def test_fused_routing_static_groups(ops, monkeypatch, T, N, used, seed):
     assert torch.equal(outs["eager"], outs["route-first"]) and torch.equal(outs["eager"], outs["planned"])
 
 
+@pytest.mark.parametrize("T,N,k,m,seed", [
+    (9000, 300, 128, 128, 91),      # more tokens than the plan kernel keeps in LDS between its passes; many deltas
+    (12000, 3, 256, 128, 92),       # long runs: hundreds of wide tiles per delta, the wide kernel takes them
+    (8300, 8192, 128, 128, 93),     # the largest delta count a plan accepts, most deltas without a token
+])
+def test_large_batches_through_the_plan(ops, T, N, k, m, seed):
+    """Batches beyond the sizes the other tests use: the plan kernel's second pass re-reads the indices
+    of tokens past its LDS cache, tile lists are thousands of entries long."""
+    say(f"large batch T={T} N={N} k={k} m={m} seed={seed}")
+    rng = np.random.default_rng(seed)
+    if N <= 300:
+        qw, meta, s = make_deltas(N, k, m, seed)
+        idx = rng.integers(-1, N, size=T).astype(np.int32)
+    else:
+        # 8192 distinct deltas would take minutes to pack: a handful of real ones, addressed through a stack
+        # whose other entries are never selected
+        real = 6
+        qw_r, meta_r, s_r = make_deltas(real, k, m, seed)
+        sel = rng.choice(N, size=real, replace=False)
+        qw = np.zeros((N,) + qw_r.shape[1:], dtype=qw_r.dtype)
+        meta = np.zeros((N,) + meta_r.shape[1:], dtype=meta_r.dtype)
+        s = np.ones((N,) + s_r.shape[1:], dtype=s_r.dtype)
+        qw[sel], meta[sel], s[sel] = qw_r, meta_r, s_r
+        idx = np.where(rng.random(T) < 0.1, -1, sel[rng.integers(0, real, size=T)]).astype(np.int32)
+    x = activations(T, k, seed + 1)
+    gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
+    out = ops.sbmm_4bit_2_4_native(gq, gx, gm, gs, gi)
+    torch.cuda.synchronize()
+    used = np.unique(idx[idx >= 0])
+    ref = np.zeros((T, m), dtype=np.float64)
+    for d in used:                                   # the oracle, one dense delta at a time
+        rows = np.nonzero(idx == d)[0]
+        ref[rows] = x[rows].astype(np.float64) @ orc.unpack(qw[d], meta[d], s[d]).astype(np.float64)
+    check_close(out, ref, what="large batch")
+    assert bool((out[torch.from_numpy(idx < 0).to(DEV)] == 0).all())
+
+
 def test_sbmm_with_base_weight_accumulates_in_place(ops):
     say("sbmm with base weight")
     T, N, k, m = 24, 4, 256, 256
