@@ -40,6 +40,7 @@ def parse():
     p.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
     p.add_argument("--tokens", type=int, default=None, help="override the token count (cfg0/cfg2/cfg3/cfg4)")
     p.add_argument("--deltas", type=int, default=None, help="override the number of resident deltas (cfg4)")
+    p.add_argument("--shape", default=None, help="K,M: override the weight shape (cfg0)")
     p.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = auto)")
     p.add_argument("--no-graph", action="store_true", help="time eager launches instead of one captured HIP graph")
     p.add_argument("--no-cpu-baseline", action="store_true")
@@ -175,7 +176,11 @@ def main():
         sys.exit(1)
     ffi.lib()   # fails loudly if the HIP library is missing
 
-    wl = W.config(a.workload, a.tokens)
+    shape = tuple(int(v) for v in a.shape.split(",")) if a.shape else None
+    if shape is not None and (a.workload != "cfg0" or len(shape) != 2 or shape[0] % 64 or shape[1] % 128):
+        print("bench.py: --shape K,M needs --workload cfg0, K % 64 == 0 and M % 128 == 0", file=sys.stderr)
+        sys.exit(2)
+    wl = W.config(a.workload, a.tokens, shape)
     if a.deltas is not None and a.workload == "cfg4":
         wl.n_deltas = a.deltas
         wl.indices = W.zipf_indices(wl.tokens, wl.n_deltas, 1.2, wl.seed)
@@ -261,7 +266,7 @@ def main():
     kflops = wl.delta_flops() / kdur / 1e12
     traffic = None
     tpath = os.path.join(ROOT, "profiles", f"traffic_{a.workload}.json")
-    if os.path.exists(tpath) and a.tokens is None and a.deltas is None:
+    if os.path.exists(tpath) and a.tokens is None and a.deltas is None and a.shape is None:
         try:
             traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
         except Exception:

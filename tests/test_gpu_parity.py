@@ -73,6 +73,7 @@ def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
     say(f"matmul {kernel} n={n} k={k} m={m} seed={seed}")
     monkeypatch.setenv("TRITEIA_HIP_WIDE_MIN_UNITS", "1")
     monkeypatch.setenv("TRITEIA_HIP_WIDE128_MIN_UNITS", "1")
+    monkeypatch.setenv("TRITEIA_HIP_WIDE128_MIN_K", "0")
     monkeypatch.setenv("TRITEIA_HIP_WIDE128", "1" if kernel == "wide128" else "0")
     qw, meta, s = make_deltas(1, k, m, seed)
     x = activations(n, k, seed + 1)

@@ -73,6 +73,20 @@ int pick_nt(long tokens, long groups) {
   return 4;
 }
 
+// Uniform groups (matmul, bmm): tokens per group are known exactly.  A launch of few workgroups is
+// bound by latency, not by the weights it re-reads from cache: the widest tile that still leaves
+// one workgroup per CU, else 16-token tiles with the tokens split across workgroups (measured on
+// one 4096 x 4096 matrix: 64 tokens 24.4 -> 12.2 us, 128 tokens 24.2 -> 12.4 us, 256 tokens 24.4 -> 19.1 us).
+int pick_nt_uniform(long tokens, long groups, long col_blocks) {
+  const int forced = env_int("TRITEIA_HIP_NT", 0);
+  if (forced == 1 || forced == 2 || forced == 4) return forced;
+  for (int nt = 4; nt >= 2; nt /= 2) {
+    if (tokens <= 8 * nt) continue;   // a narrower tile holds them all
+    if (groups * col_blocks * ((tokens + 16 * nt - 1) / (16 * nt)) >= 256) return nt;
+  }
+  return 1;
+}
+
 template <int NT, int KW, int DEPTH, bool EAGER = false>
 void launch_one(const Sparse24Args& a, dim3 grid, hipStream_t st) {
   hipLaunchKernelGGL((sparse24_grouped_kernel<NT, KW, DEPTH, EAGER>), grid, dim3(64 * KW), 0, st, a);
@@ -85,7 +99,14 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   if (tsplit < 1) tsplit = 1;
   if (tsplit > 65535) tsplit = 65535;
   const long cb_pad = (a.m / 128 + 7) / 8 * 8;   // column blocks padded to the 8 XCDs
-  const int kw = env_int("TRITEIA_HIP_KW", 4);
+  // A launch of at most one workgroup per CU runs 8 wavefronts per workgroup with one step in
+  // flight each: more waves, not more bytes per wave, is what raises the rate there (measured:
+  // cfg1 14.3 -> 13.6 us, 16-token matmul 12.3 -> 11.4 us; 16 wavefronts and two steps per wave are slower).
+  // Only for uniform groups (matmul, bmm): the split of K among the wavefronts fixes the order of the
+  // fp32 sums, and a routed token must have the same bits whatever the size of its batch.
+  const bool uniform = !a.raw_indices && !a.tiles && !a.g_delta;
+  const bool one_per_cu = uniform && (nt == 1 || nt == 2) && (long)a.n_groups * cb_pad * tsplit <= 256;
+  const int kw = env_int("TRITEIA_HIP_KW", one_per_cu ? 8 : 4);
   // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight (2 with
   // two), the 32-token kernel 2 per CU with two, the 64-token kernel 1 per CU with one.  Fused
   // routing in its eager form keeps one step in flight (measured: a second step requested ahead of
@@ -95,7 +116,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   // of each wave's chain of requests rather than by bandwidth: a second step in flight pays there
   // (5-12 % measured) while it costs time on full launches
   const bool small = (long)a.n_groups * cb_pad * tsplit <= 512;
-  const int depth = env_int("TRITEIA_HIP_DEPTH", eager ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1));
+  const int depth = env_int("TRITEIA_HIP_DEPTH", eager || kw == 8 ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1));
   if (eager && !(kw == 4 && ((nt == 1 && depth == 2) || (nt == 1 && depth == 1) || (nt == 2 && depth == 1) || (nt == 4 && depth == 1)))) {
     a.raw_static = 0;   // no eager build of this variant: route first, then request
     a.n_groups = a.raw_count < a.n_deltas ? a.raw_count : a.n_deltas;
@@ -117,7 +138,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   if (a.raw_indices && a.raw_static) {
     TRY_EAGER(1, 4, 1) TRY_EAGER(1, 4, 2) TRY_EAGER(2, 4, 1) TRY_EAGER(4, 4, 1)
   }
-  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 2)
+  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 1) TRY(1, 8, 2)
   TRY(2, 4, 1) TRY(2, 4, 2) TRY(2, 8, 1)
   TRY(4, 4, 1)
 #undef TRY
@@ -215,7 +236,9 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   int done = 0;
   // (the 128-token kernel addresses activations with 32-bit byte offsets)
   const bool x_below_4g = ((long)(n_groups - 1) * stride + tokens) * a.x_stride * 2 < (1L << 32);
-  if (wide128_enabled() && a.k % 128 == 0 && x_below_4g &&
+  // (the 128-token kernel pays from k = 8192 on: 2-3 % faster than the 64-token kernel at 8192 x 8192 and
+  // 8192 x 28672, 4-8 % slower at 4096 x 4096 and 4096 x 11008, whose K loops are too short for its pipeline)
+  if (wide128_enabled() && a.k % 128 == 0 && a.k >= env_int("TRITEIA_HIP_WIDE128_MIN_K", 8192) && x_below_4g &&
       (long)n_groups * (tokens / kWide128Tokens) * cgs >= env_int("TRITEIA_HIP_WIDE128_MIN_UNITS", kWide128MinUnits)) {
     int t = tokens / kWide128Tokens * kWide128Tokens;
     if (tokens - t > kWideTokens) t = tokens;
@@ -239,7 +262,7 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   if (rest > 0) {
     a.uniform_first = done;
     a.uniform_count = rest;
-    const int nt = pick_nt(rest, 1);
+    const int nt = pick_nt_uniform(rest, n_groups, a.m / 128);
     return launch_sparse24(a, nt, (rest + 16 * nt - 1) / (16 * nt), st);
   }
   return TRITEIA_HIP_OK;

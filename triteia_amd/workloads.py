@@ -88,11 +88,13 @@ class Workload:
         return b
 
 
-def config(name, tokens=None):
-    """The five benchmark configurations (seed = 1000 + index)."""
+def config(name, tokens=None, shape=None):
+    """The five benchmark configurations (seed = 1000 + index).  `shape` = (k, m) overrides the weight
+    shape of cfg0 (the single-matrix op at other layer shapes)."""
     if name == "cfg0":
         t = 16 if tokens is None else tokens
-        return Workload(f"cfg0 matmul_4bit_2_4 x[{t},4096] W[4096x4096]", "matmul", 4096, 4096, 1, t, 1000)
+        k, m = (4096, 4096) if shape is None else shape
+        return Workload(f"cfg0 matmul_4bit_2_4 x[{t},{k}] W[{k}x{m}]", "matmul", k, m, 1, t, 1000)
     if name == "cfg1":
         return Workload("cfg1 bmm_4bit_2_4 8 deltas 4096x4096, 1 token each", "bmm", 4096, 4096, 8, 8, 1001)
     if name == "cfg2":
