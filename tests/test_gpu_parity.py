@@ -351,6 +351,36 @@ def test_large_batches_through_the_plan(ops, T, N, k, m, seed):
     assert bool((out[torch.from_numpy(idx < 0).to(DEV)] == 0).all())
 
 
+@pytest.mark.parametrize("T,N,k,m,seed", [(64, 1, 512, 384, 95), (150, 2, 256, 640, 96), (100, 1, 320, 128, 97)])
+def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, m, seed):
+    """One or two deltas with tens of tokens on a narrow layer: the plan's 64-token tiles are taken in
+    16-token passes split over workgroups.  Same bits as whole tiles (the order of the sums over K does not
+    depend on the pass width), within the bar of the oracle."""
+    say(f"few deltas T={T} N={N} k={k} m={m} seed={seed}")
+    from triteia_amd.python.capi import sbmm_2_4_routed
+    qw, meta, s = make_deltas(N, k, m, seed)
+    x = activations(T, k, seed + 1)
+    idx = np.random.default_rng(seed + 2).integers(-1, N, size=T).astype(np.int32)
+    ref = orc.sbmm_4bit_2_4(qw, x, meta, s, idx)
+    gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
+    outs = []
+    for passes in ("4", "2", "1", None):
+        monkeypatch.setenv("TRITEIA_HIP_FUSED_ROUTE", "0")
+        if passes is None:
+            monkeypatch.delenv("TRITEIA_HIP_PASS_NT", raising=False)
+        else:
+            monkeypatch.setenv("TRITEIA_HIP_PASS_NT", passes)
+        out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
+        sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
+        torch.cuda.synchronize()
+        outs.append(out)
+    none = torch.from_numpy(idx < 0).to(DEV)
+    assert bool((outs[0][none] == -3.0).all())
+    check_close(torch.where(none[:, None], torch.zeros_like(outs[0]), outs[0]), ref, what="split passes")
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+
+
 def test_sbmm_with_base_weight_accumulates_in_place(ops):
     say("sbmm with base weight")
     T, N, k, m = 24, 4, 256, 256

@@ -408,7 +408,21 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     wide_launch = prob_k % 128 == 0 && (long)(prob_n / 48 + 1) * a.wide_gate >= a.wide_min_units;
     if (!wide_launch) a.wide_min_units = 0x7fffffff;
   }
-  if (int e = launch_sparse24(a, tile / 16, 1, static_cast<hipStream_t>(stream))) return e;
+  // The plan's tiles are cut without knowledge of the layer.  Where they make a launch of very few
+  // workgroups on this layer (one or two deltas, a narrow matrix: fewer than 200 even on the plan's
+  // upper bound of tiles), the kernel takes them in narrower passes split over workgroups (the weights
+  // re-read that way come from cache) until there is a workgroup per CU.  Measured on 4096 x 4096: one
+  // delta with 64 / 128 tokens 24.4 -> 12.7 / 24.2 -> 18.8 us, two deltas with 256 tokens 24.6 -> 18.5 us;
+  // launches of 250 workgroups and more lose 10 % that way and keep the plan's tile.
+  int pass_nt = tile / 16;
+  {
+    const long cb_pad = (prob_m / 128 + 7) / 8 * 8;
+    if ((long)a.n_groups * cb_pad < 200)
+      while (pass_nt > 1 && (long)a.n_groups * cb_pad * (tile / (16 * pass_nt)) < 256) pass_nt /= 2;
+    const int forced = env_int("TRITEIA_HIP_PASS_NT", 0);
+    if ((forced == 1 || forced == 2 || forced == 4) && 16 * forced <= tile) pass_nt = forced;
+  }
+  if (int e = launch_sparse24(a, pass_nt, tile / (16 * pass_nt), static_cast<hipStream_t>(stream))) return e;
   if (wide_launch) {
     a.tiles = reinterpret_cast<const int4*>(ws + L.wide);
     a.tiles_alt = nullptr;
