@@ -74,6 +74,7 @@ class Problem:
             self.lora_a = (torch.randn((wl.n_lora, wl.k, wl.lora_rank), generator=g, device=dev) * 0.01).half()
             self.lora_b = (torch.randn((wl.n_lora, wl.lora_rank, wl.m), generator=g, device=dev) * 0.01).half()
             self.v = torch.zeros((wl.tokens, wl.lora_rank), dtype=torch.float16, device=dev)
+            self.side = torch.cuda.Stream(device=dev)      # default priority
 
     def _chk(self, rc):
         if rc != 0:
@@ -111,13 +112,26 @@ class Problem:
             self._chk(self.lib.triteia_hip_sbmm_2_4_routed(P(self.x), P(q), P(me), P(self.out), P(s), P(self.idx), 0, wl.n_deltas, wl.m,
                                                            wl.tokens, wl.k, P(self.ws), self.ws_bytes, 0, 0, self.stream()))
         else:  # ldmm: dense base GEMM (library) + routed LoRA (SGMV) + routed delta, one routing plan for both
-            torch.matmul(self.x, self.base[i % self.copies].t(), out=self.out)
-            self.plan()
-            self.v.zero_()
-            st = self.stream()
             r = wl.lora_rank
-            self._chk(self.lib.triteia_hip_sgmv_routed(P(self.v), r, P(self.x), wl.k, P(self.lora_a), wl.k * r, wl.n_lora, wl.k, r,
-                                                       1.0, P(self.ws), wl.tokens, 0, st))
+            cur = torch.cuda.current_stream()
+            side = self.side if os.environ.get("BENCH_LDMM_OVERLAP", "1") == "1" else None
+            if side is not None:
+                # routing and the LoRA shrink need only x: they run beside the base GEMM, which leaves CUs idle
+                side.wait_stream(cur)
+                with torch.cuda.stream(side):
+                    self.plan()
+                    self.v.zero_()
+                    self._chk(self.lib.triteia_hip_sgmv_routed(P(self.v), r, P(self.x), wl.k, P(self.lora_a), wl.k * r, wl.n_lora,
+                                                               wl.k, r, 1.0, P(self.ws), wl.tokens, 0, self.stream()))
+                torch.matmul(self.x, self.base[i % self.copies].t(), out=self.out)
+                cur.wait_stream(side)
+            else:
+                torch.matmul(self.x, self.base[i % self.copies].t(), out=self.out)
+                self.plan()
+                self.v.zero_()
+                self._chk(self.lib.triteia_hip_sgmv_routed(P(self.v), r, P(self.x), wl.k, P(self.lora_a), wl.k * r, wl.n_lora, wl.k, r,
+                                                           1.0, P(self.ws), wl.tokens, 0, self.stream()))
+            st = self.stream()
             self._chk(self.lib.triteia_hip_sgmv_routed(P(self.out), wl.m, P(self.v), r, P(self.lora_b), r * wl.m, wl.n_lora, r, wl.m,
                                                        1.0, P(self.ws), wl.tokens, 0, st))
             self.delta_kernel(i, accumulate=1)

@@ -515,3 +515,14 @@ def test_ldmm(ops, T, M, N, m, k, r, seed):
     only_delta = ops.sbmm_4bit_2_4_native(gq, gx, gm, gs, torch.where(gi >= M, gi - M, -1).int())
     rows = torch.from_numpy(idx >= M).to(DEV)
     assert torch.equal(out[rows], only_delta[rows])
+    # with a dense base weight (routing and the LoRA shrink then run on a side stream beside the base GEMM):
+    # the library GEMM's fp16 result is taken as given, the routed parts are added to it in place
+    base_w = (np.random.default_rng(seed + 4).standard_normal((m, k)) * 0.02).astype(np.float16)
+    gb = torch.from_numpy(base_w).to(DEV)
+    for _ in range(3):                                   # several calls in a row share the side stream
+        with_base = ops.ldmm(gi, gx, gA, gB, gq, gm, gs, base_weight=gb)
+    torch.cuda.synchronize()
+    y0 = torch.matmul(gx, gb.t())
+    ref_b = y0.float().cpu().numpy().astype(np.float64) + ref
+    check_close(with_base, ref_b, what="ldmm + base")
+    assert torch.equal(with_base[torch.from_numpy(idx < 0).to(DEV)], y0[torch.from_numpy(idx < 0).to(DEV)])

@@ -5,9 +5,20 @@ delta indices[t] - M; -1 means base model only.
 """
 import torch
 
-from triteia_amd.python.capi import route_plan, sbmm_2_4_routed, sgmv_routed
+from triteia_amd.python.capi import route_plan, routed_workspace, sbmm_2_4_routed, sgmv_routed
 from .lora import lora_forloop
 from .sbmm import sbmm_4bit_2_4_forloop
+
+
+_SIDE_STREAMS = {}
+
+
+def _side_stream(device):
+    """One extra stream per device (default priority), made at first use."""
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    if key not in _SIDE_STREAMS:
+        _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
+    return _SIDE_STREAMS[key]
 
 
 def baseline_ldmm(indices, x, LwA, LwB, DeltaW, metas, ss, base_weight=None, debug=False):
@@ -41,18 +52,36 @@ def ldmm(indices, x, LwA, LwB, DeltaW, metas, ss, base_weight=None, debug=False)
     packed deltas.  Returns [B, H2] in x.dtype."""
     x_ = x.to(torch.float16)
     x_ = x_ if x_.is_contiguous() else x_.contiguous()
-    if base_weight is not None:
-        y = torch.matmul(x_, base_weight.t())
-    else:
-        y = torch.zeros(x_.shape[0], LwB.shape[2], dtype=x_.dtype, device=x_.device)
     M = LwA.shape[0]
     idx32 = indices.to(torch.int32)
     if M > 0:
-        # the plan over M adapters skips -1 and every index >= M (the delta tokens)
-        plan = route_plan(idx32, M)
-        v = torch.zeros((x_.shape[0], LwA.shape[2]), dtype=torch.float16, device=x_.device)
-        sgmv_routed(v, x_, LwA.to(torch.float16).contiguous(), plan)
-        sgmv_routed(y, v, LwB.to(torch.float16).contiguous(), plan)
+        A16, B16 = LwA.to(torch.float16).contiguous(), LwB.to(torch.float16).contiguous()
+        ws = routed_workspace(x_.shape[0], M, x_.device)
+        v = torch.empty((x_.shape[0], LwA.shape[2]), dtype=torch.float16, device=x_.device)
+    if M > 0 and base_weight is not None:
+        # Routing and the LoRA shrink need only x: they run on a side stream beside the base GEMM (a
+        # library GEMM of a few hundred tokens leaves CUs idle) and join before the expand.  All
+        # buffers are allocated on the current stream, which also frees them.
+        cur = torch.cuda.current_stream(x_.device)
+        side = _side_stream(x_.device)
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):
+            plan = route_plan(idx32, M, workspace=ws)      # skips -1 and every index >= M (the delta tokens)
+            v.zero_()
+            sgmv_routed(v, x_, A16, plan)
+        y = torch.matmul(x_, base_weight.t())
+        cur.wait_stream(side)
+        sgmv_routed(y, v, B16, plan)
+    else:
+        if base_weight is not None:
+            y = torch.matmul(x_, base_weight.t())
+        else:
+            y = torch.zeros(x_.shape[0], LwB.shape[2], dtype=x_.dtype, device=x_.device)
+        if M > 0:
+            plan = route_plan(idx32, M, workspace=ws)
+            v.zero_()
+            sgmv_routed(v, x_, A16, plan)
+            sgmv_routed(y, v, B16, plan)
     if DeltaW.shape[0] > 0:
         sbmm_2_4_routed(x_, DeltaW, metas, y, ss, idx32, index_offset=M, accumulate=True)
     return y.to(x.dtype)
