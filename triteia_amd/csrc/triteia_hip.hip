@@ -222,7 +222,7 @@ int launch_wide128(const Sparse24Args& a, hipStream_t st) {
 // the 128-token one; TRITEIA_HIP_WIDE_MIN_UNITS / TRITEIA_HIP_WIDE128_MIN_UNITS move the thresholds.
 bool wide_enabled() { return env_int("TRITEIA_HIP_WIDE", 1) != 0; }
 bool wide128_enabled() { return wide_enabled() && env_int("TRITEIA_HIP_WIDE128", 1) != 0; }
-constexpr long kWideMinUnits = 128;
+constexpr long kWideMinUnits = 160;   // 4096 x 4096: 1024 tokens (128 tiles) 54.9 us wide against 46.5 us narrow, 1536 tokens (192) 60.8 against 71.1
 constexpr long kWide128MinUnits = 192;
 
 // `tokens` rows per group, `stride` rows between groups: the head of each group goes to the
