@@ -381,6 +381,38 @@ def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, 
         assert torch.equal(o, outs[0])
 
 
+def test_empty_and_degenerate_inputs(ops):
+    """Zero tokens, zero deltas, zero adapters, a batch in which nothing is routed: every op returns the
+    shape it should and touches nothing else."""
+    say("empty and degenerate inputs")
+    N, k, m, r = 3, 256, 256, 16
+    qw, meta, s = make_deltas(N, k, m, 98)
+    A, B = _lora_weights(2, k, r, m, 99, scale=0.05)
+    gq, gm, gs, gA, gB = to_gpu(qw, meta, s, A, B)
+    x0 = torch.zeros((0, k), dtype=torch.float16, device=DEV)
+    i0 = torch.zeros((0,), dtype=torch.int32, device=DEV)
+    assert ops.matmul_4bit_2_4(gq[0], x0, gm[0], gs[0]).shape == (0, m)
+    assert ops.sbmm_4bit_2_4_native(gq, x0, gm, gs, i0).shape == (0, m)
+    assert ops.sbmm_4bit_2_4_forloop(gq, x0, gm, gs, i0).shape == (0, m)
+    assert ops.lora_sgmv_routed(gA, gB, x0, i0).shape == (0, m)
+    assert ops.lora_bgmv(gA, gB, x0, i0).shape == (0, m)
+    assert ops.ldmm(i0, x0, gA, gB, gq, gm, gs).shape == (0, m)
+    assert ops.bmm_4bit_2_4(gq[:0], torch.zeros((0, 4, k), dtype=torch.float16, device=DEV), gm[:0], gs[:0]).shape == (0, 4, m)
+    # tokens, but no delta / adapter selected
+    x = torch.from_numpy(activations(70, k, 100)).to(DEV)
+    none = torch.full((70,), -1, dtype=torch.int32, device=DEV)
+    for T in (5, 70):
+        assert bool((ops.sbmm_4bit_2_4_native(gq, x[:T], gm, gs, none[:T]) == 0).all())
+        assert bool((ops.lora_sgmv_routed(gA, gB, x[:T], none[:T]) == 0).all())
+        assert bool((ops.ldmm(none[:T], x[:T], gA, gB, gq, gm, gs) == 0).all())
+    # no LoRA adapters at all: ldmm is the routed delta op
+    idx = torch.from_numpy(np.random.default_rng(101).integers(-1, N, size=70).astype(np.int32)).to(DEV)
+    noA = torch.zeros((0, k, r), dtype=torch.float16, device=DEV)
+    noB = torch.zeros((0, r, m), dtype=torch.float16, device=DEV)
+    assert torch.equal(ops.ldmm(idx, x, noA, noB, gq, gm, gs), ops.sbmm_4bit_2_4_native(gq, x, gm, gs, idx))
+    torch.cuda.synchronize()
+
+
 def test_sbmm_with_base_weight_accumulates_in_place(ops):
     say("sbmm with base weight")
     T, N, k, m = 24, 4, 256, 256
