@@ -253,7 +253,7 @@ def _exact_problem(T, N, k, m, seed):
 
 
 @pytest.mark.parametrize("T,N,k,m,seed", [(64, 16, 512, 384, 51), (37, 5, 1024, 256, 52), (300, 7, 512, 640, 53), (700, 3, 256, 512, 54),
-                                          (128, 16, 512, 256, 55), (97, 3, 256, 384, 56)])
+                                          (128, 16, 512, 256, 55), (97, 3, 256, 384, 56), (256, 32, 256, 256, 60), (193, 2, 512, 128, 61)])
 def test_routing_is_bit_exact_on_exact_arithmetic(ops, monkeypatch, T, N, k, m, seed):
     """With inputs on which floating point is exact, every path (fused routing, routing plan with narrow
     and wide tiles, run table, one launch per run, one matmul per delta) must reproduce the oracle bit
@@ -287,11 +287,16 @@ def test_routing_is_bit_exact_on_exact_arithmetic(ops, monkeypatch, T, N, k, m, 
     (128, 16, list(range(16)), 45),      # two tokens per lane: groups that span both halves of the batch
     (100, 8, [1, 2, 6], 46),             # ... with a ragged second half and 30-token groups (two 16-token passes)
     (70, 40, [3, 39], 47),               # ... routing first
-    (128, 64, list(range(64)), 48),      # as many deltas as a wavefront has lanes
+    (128, 32, list(range(32)), 48),      # the most deltas this form takes above 64 tokens
+    (64, 64, list(range(64)), 62),       # as many deltas as a wavefront has lanes
     (65, 2, [0, 1], 49),                 # one token in the second half
+    (256, 16, list(range(16)), 50),      # four tokens per lane
+    (200, 32, list(range(0, 32, 3)), 57),
+    (129, 4, [0, 3], 58),                # one token in the third part
+    (250, 3, [1], 59),                   # one delta takes nearly everything: 13 passes of 16 tokens / 4 of 64
 ])
 def test_fused_routing_static_groups(ops, monkeypatch, T, N, used, seed):
-    """Batches of at most 128 tokens are routed inside the multiply kernel; with at least two tokens per
+    """Batches of at most 256 tokens are routed inside the multiply kernel; with at least two tokens per
     delta every delta is a group of its own and its first weights are requested before the indices
     have arrived.  Same bits as routing first (TRITEIA_HIP_EAGER=0) and as the plan-based path."""
     say(f"fused routing T={T} N={N} used={used} seed={seed}")

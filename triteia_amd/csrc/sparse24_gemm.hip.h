@@ -67,7 +67,7 @@ struct Sparse24Args {
   //   g_*     : three separate arrays (the reference's run table)
   //   none    : group j = delta j*delta_step with uniform_count rows from
   //             j*uniform_stride + uniform_first
-  //   raw_indices : (takes precedence) the batch's per-token delta indices, at most 128 tokens
+  //   raw_indices : (takes precedence) the batch's per-token delta indices, at most 256 tokens
   //             and 64 deltas: every workgroup derives its group itself ("fused routing"),
   //             group j = the j-th delta in use, in ascending order
   const int4* tiles;
@@ -161,6 +161,8 @@ struct WPre {
   uint4_t mt[2];
 };
 
+constexpr int kRawParts = 4;     // fused routing: tokens per lane, i.e. batches of up to 256 tokens
+
 constexpr int kRedStride = 132;  // floats per token row in the reduction buffer (128 + pad)
 
 // Everything one workgroup knows about its (group, column block) before touching tokens.
@@ -173,9 +175,12 @@ struct TileCtx {
   int rot;                  // this delta's walk over K starts at step `rot` and wraps around
   int cb;                   // column block
   int tid, wave, lane, r, q;
-  int raw_list;             // fused routing: lane s holds the s-th of the group's tokens among tokens 0..63 ...
-  int raw_list2;            // ... and among tokens 64..127 (slots of the group: first those, then these)
-  int raw_first_half;       // how many of the group's tokens lie among tokens 0..63
+  // fused routing (up to kRawParts x 64 tokens, kRawParts per lane): for part j of the batch (tokens
+  // 64 j .. 64 j + 63), lane s of raw_list[j] holds the s-th of the group's tokens in that part, and
+  // raw_before[j] counts the group's tokens in the parts before it.  The group's slots run through
+  // the parts in order.
+  int raw_list[kRawParts];
+  int raw_before[kRawParts + 1];
   half8_t sv;               // scales of this thread's 8 output features (requested at start-up)
 #ifdef TRITEIA_HIP_TIMELINE
   long long ts[4];          // debug builds: entry, operands requested, K loop done, end
@@ -221,9 +226,13 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
     const int slot = min(nt * 16 + r, cnt - 1);   // slots past the end re-read the last row
     if (p.raw_indices) {
       const int sigma = first + slot;
-      const int lo = __shfl(c.raw_list, sigma, 64);
-      const int hi = __shfl(c.raw_list2, sigma - c.raw_first_half, 64);
-      rows[nt] = sigma < c.raw_first_half ? lo : hi;
+      int row = 0;
+#pragma unroll
+      for (int j = 0; j < kRawParts; j++) {
+        const int v = __shfl(c.raw_list[j], sigma - c.raw_before[j], 64);
+        if (sigma >= c.raw_before[j] && sigma < c.raw_before[j + 1]) row = v;
+      }
+      rows[nt] = row;
     } else rows[nt] = p.perm ? p.perm[first + slot] : first + slot;
   }
   StepFrag<NTT> ring[DEPTH];
@@ -417,9 +426,9 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   c.r = c.lane & 15;
   c.q = c.lane >> 4;
   c.cb = cb;
-  c.raw_list = 0;
-  c.raw_list2 = 0;
-  c.raw_first_half = 0;
+#pragma unroll
+  for (int j = 0; j < kRawParts; j++) c.raw_list[j] = c.raw_before[j] = 0;
+  c.raw_before[kRawParts] = 0;
   c.k_rows = p.k >> 5;                 // packed rows (32 dense k each)
   c.n_steps = (c.k_rows + 3) >> 2;     // 128 dense k per step
   c.qrow = p.m >> 1;
@@ -444,9 +453,9 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
     // Fused routing for small batches: every wavefront looks at all (<= 64) indices, one per
     // lane, and works out its delta and the rows routed to it -- a few dozen instructions
     // instead of a separate routing launch and a dependent descriptor read.
-    int d = -1, d2 = -1;     // this lane's two tokens: lane and 64 + lane
-    if (c.lane < p.raw_count) d = p.raw_indices[c.lane];
-    if (c.lane + 64 < p.raw_count) d2 = p.raw_indices[c.lane + 64];
+    int d[kRawParts];     // this lane's tokens: lane, 64 + lane, ...
+#pragma unroll
+    for (int j = 0; j < kRawParts; j++) d[j] = (64 * j + c.lane < p.raw_count) ? p.raw_indices[64 * j + c.lane] : -1;
     if (EAGER) {
       // group g is delta g: its first weights are requested right behind the indices
       if (grp >= p.n_deltas) return;
@@ -469,14 +478,17 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
       // nothing that needs the indices may be scheduled (with its wait) ahead of these requests
       __builtin_amdgcn_sched_barrier(0);
     }
-    d -= p.raw_offset;
-    d2 -= p.raw_offset;
-    if (c.lane >= p.raw_count || d < 0 || d >= p.n_deltas) d = -1;
-    if (c.lane + 64 >= p.raw_count || d2 < 0 || d2 >= p.n_deltas) d2 = -1;
+#pragma unroll
+    for (int j = 0; j < kRawParts; j++) {
+      const int v = d[j] - p.raw_offset;
+      d[j] = (64 * j + c.lane < p.raw_count && v >= 0 && v < p.n_deltas) ? v : -1;
+    }
     const unsigned long long below = (1ull << c.lane) - 1ull;
     if (!EAGER) {
       // the grp-th delta in use
-      unsigned long long used = (d >= 0 ? (1ull << d) : 0ull) | (d2 >= 0 ? (1ull << d2) : 0ull);
+      unsigned long long used = 0ull;
+#pragma unroll
+      for (int j = 0; j < kRawParts; j++) used |= d[j] >= 0 ? (1ull << d[j]) : 0ull;
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) {
         const unsigned lo = __shfl_xor((unsigned)used, off, 64);
@@ -487,21 +499,21 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
       const bool is_grp = ((used >> c.lane) & 1ull) && __popcll(used & below) == grp;
       delta = __ffsll((long long)__ballot(is_grp)) - 1;
     }
-    const unsigned long long members = __ballot(d == delta);
-    const unsigned long long members2 = __ballot(d2 == delta);
-    const int c1 = __popcll(members), c2 = __popcll(members2);
-    count = c1 + c2;
+    // slot s of the group = its s-th member token.  Per part of the batch, a full permutation sends
+    // every member's token id to the lane of its rank (non-members fill the lanes after the members)
+    count = 0;
     start = 0;
-    // slot s of the group = its s-th member token.  Per half of the batch, a full permutation sends
-    // every member's token id to the lane of its rank (non-members fill the lanes after the members);
-    // the group's slots are the members of the first half followed by those of the second.
-    const int rank = __popcll(members & below);
-    const int dest = (d == delta) ? rank : c1 + (c.lane - rank);
-    c.raw_list = __builtin_amdgcn_ds_permute(dest << 2, c.lane);
-    const int rank2 = __popcll(members2 & below);
-    const int dest2 = (d2 == delta) ? rank2 : c2 + (c.lane - rank2);
-    c.raw_list2 = __builtin_amdgcn_ds_permute(dest2 << 2, c.lane + 64);
-    c.raw_first_half = c1;
+#pragma unroll
+    for (int j = 0; j < kRawParts; j++) {
+      const unsigned long long members = __ballot(d[j] == delta);
+      const int cj = __popcll(members);
+      const int rank = __popcll(members & below);
+      const int dest = (d[j] == delta) ? rank : cj + (c.lane - rank);
+      c.raw_list[j] = __builtin_amdgcn_ds_permute(dest << 2, 64 * j + c.lane);
+      c.raw_before[j] = count;
+      count += cj;
+    }
+    c.raw_before[kRawParts] = count;
     if (EAGER && count <= 0) {
       __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): let the requested weights land before the wave ends
       return;

@@ -352,7 +352,7 @@ int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas) {
 // layer >= kPlanWideMinUnits); otherwise re-reading a hot delta's weights from cache in narrow
 // tiles is cheaper than a second, poorly filled launch, and the wide launch returns at once.
 constexpr int kPlanWideMinUnits = 200;
-constexpr int kFusedMaxTokens = 128;   // two tokens per lane of a wavefront
+constexpr int kFusedMaxTokens = 64 * kRawParts;   // kRawParts tokens per lane of a wavefront
 static int plan_has_wide(int prob_n, int n_deltas) {
   const long groups = n_deltas < prob_n ? n_deltas : prob_n;
   return wide_enabled() && prob_n >= env_int("TRITEIA_HIP_WIDE_MIN_BATCH", 256) && prob_n >= 8 * groups;
@@ -442,8 +442,10 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: accumulate=%d", accumulate);
   if (prob_m == 0 || prob_n == 0 || prob_k == 0 || n_deltas == 0) return TRITEIA_HIP_OK;
   if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null tensor pointer");
-  if (prob_n <= env_int("TRITEIA_HIP_FUSED_MAX_TOKENS", kFusedMaxTokens) && prob_n <= kFusedMaxTokens && n_deltas <= 64 &&
-      env_int("TRITEIA_HIP_FUSED_ROUTE", 1)) {
+  // (above 64 tokens only for at most 32 deltas: with 64 deltas of 8192 x 28672 under a skewed routing the
+  // workgroups of the deltas without tokens make this form 1-2 % slower than a plan, which lists none)
+  if (prob_n <= env_int("TRITEIA_HIP_FUSED_MAX_TOKENS", kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
+      n_deltas <= (prob_n > 64 ? 32 : 64) && env_int("TRITEIA_HIP_FUSED_ROUTE", 1)) {
     // small batch: the multiply kernel routes by itself, no plan, no workspace traffic
     if (!token_indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null indices");
     DeviceGuard g(dev);
@@ -459,8 +461,7 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
     // With at least two tokens per delta on average nearly every delta is in use: one group per
     // delta, whose weights are requested before the indices have arrived (a delta without
     // tokens costs one prefetched step per wave).  Sparser batches route first.
-    // (four per delta for batches above 64 tokens: measured on 64 deltas of 8192 x 28672 under a skewed
-    // routing of 128 tokens, 35 deltas in use: 544 us eager against 526 us routing first)
+    // (four per delta for batches above 64 tokens)
     if (prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && env_int("TRITEIA_HIP_EAGER", 1)) {
       a.raw_static = 1;
       a.n_groups = n_deltas;
