@@ -461,8 +461,10 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
     // With at least two tokens per delta on average nearly every delta is in use: one group per
     // delta, whose weights are requested before the indices have arrived (a delta without
     // tokens costs one prefetched step per wave).  Sparser batches route first.
-    // (four per delta for batches above 64 tokens)
-    if (prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && env_int("TRITEIA_HIP_EAGER", 1)) {
+    // (four per delta for batches above 64 tokens).  Only for at most 16 deltas: under a skewed routing
+    // larger sets leave many deltas without a token (Zipf(1.5) over 32: 14 in use at 64 tokens, and the
+    // prefetched steps of the other 18 make the launch 10 % slower than routing first).
+    if (n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && env_int("TRITEIA_HIP_EAGER", 1)) {
       a.raw_static = 1;
       a.n_groups = n_deltas;
     }
