@@ -255,9 +255,10 @@ def main():
     value = flops / (elapsed / a.steps) / 1e12
 
     # ---- dominant kernel alone: HIP events on the launch stream, batches of back-to-back launches
-    # (a batch of at most 64 tokens over at most 64 deltas is routed inside the multiply kernel: the whole
-    # step is that one launch, and it is the kernel timed here; otherwise the multiply runs on a routing plan)
-    fused = wl.op == "sbmm" and wl.tokens <= 64 and wl.n_deltas <= 64
+    # (a batch of at most 64 tokens over at most 64 deltas, or of at most 256 tokens over at most 32 deltas,
+    # is routed inside the multiply kernel: the whole step is that one launch, and it is the kernel timed
+    # here; otherwise the multiply runs on a routing plan)
+    fused = wl.op == "sbmm" and ((wl.tokens <= 64 and wl.n_deltas <= 64) or (wl.tokens <= 256 and wl.n_deltas <= 32))
     kernel_call = prob.step if fused else prob.delta_kernel
     if wl.indices is not None and not fused:
         prob.plan()

@@ -162,20 +162,7 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.m = prob_m;
   a.k = prob_k;
   a.n_deltas = n_deltas;
-  a.tiles = nullptr;
-  a.raw_indices = nullptr;
-  a.raw_count = 0;
-  a.raw_offset = 0;
-  a.raw_static = 0;
-  a.g_delta = a.g_start = a.g_count = a.perm = a.n_groups_dev = nullptr;
-  a.n_groups = 0;
-  a.uniform_count = 0;
-  a.uniform_stride = 0;
-  a.uniform_first = 0;
-  a.delta_step = 0;
-  a.accumulate = 0;
   a.xcd_swizzle = env_int("TRITEIA_HIP_XCD_SWIZZLE", 1);
-  a.rot_spread = 0;
 #ifdef TRITEIA_HIP_TIMELINE
   a.timeline = reinterpret_cast<long long*>(strtoull(getenv("TRITEIA_HIP_TIMELINE_PTR") ? getenv("TRITEIA_HIP_TIMELINE_PTR") : "0", nullptr, 0));
 #endif
@@ -458,12 +445,12 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
     a.n_groups = prob_n < n_deltas ? prob_n : n_deltas;
     a.accumulate = accumulate;
     const int nt = pick_nt(prob_n, a.n_groups);
-    // With at least two tokens per delta on average nearly every delta is in use: one group per
-    // delta, whose weights are requested before the indices have arrived (a delta without
-    // tokens costs one prefetched step per wave).  Sparser batches route first.
-    // (four per delta for batches above 64 tokens).  Only for at most 16 deltas: under a skewed routing
-    // larger sets leave many deltas without a token (Zipf(1.5) over 32: 14 in use at 64 tokens, and the
-    // prefetched steps of the other 18 make the launch 10 % slower than routing first).
+    // With at least two tokens per delta on average (four for batches above 64 tokens) nearly every
+    // delta is in use: one group per delta, whose weights are requested before the indices have
+    // arrived (a delta without tokens costs one prefetched step per wave).  Sparser batches route
+    // first.  Only for at most 16 deltas: under a skewed routing larger sets leave many deltas
+    // without a token (Zipf(1.5) over 32: 14 in use at 64 tokens, and the prefetched steps of the
+    // other 18 make the launch 10 % slower than routing first).
     if (n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && env_int("TRITEIA_HIP_EAGER", 1)) {
       a.raw_static = 1;
       a.n_groups = n_deltas;
