@@ -60,7 +60,7 @@ def ldmm(indices, x, LwA, LwB, DeltaW, metas, ss, base_weight=None, debug=False)
         v = torch.empty((x_.shape[0], LwA.shape[2]), dtype=torch.float16, device=x_.device)
     if M > 0 and base_weight is not None:
         # Routing and the LoRA shrink need only x: they run on a side stream beside the base GEMM (a
-        # library GEMM of a few hundred tokens leaves CUs idle) and join before the expand.  All
+        # library GEMM of a few hundred tokens leaves CUs idle); the expand follows the GEMM.  All
         # buffers are allocated on the current stream, which also frees them.
         cur = torch.cuda.current_stream(x_.device)
         side = _side_stream(x_.device)
@@ -70,6 +70,15 @@ def ldmm(indices, x, LwA, LwB, DeltaW, metas, ss, base_weight=None, debug=False)
             v.zero_()
             sgmv_routed(v, x_, A16, plan)
         y = torch.matmul(x_, base_weight.t())
+        if DeltaW.shape[0] > 0:
+            # LoRA tokens and delta tokens are different rows of y (disjoint index ranges): the expand stays
+            # on the side stream, beside the delta kernel, and joins at the end
+            side.wait_stream(cur)
+            with torch.cuda.stream(side):
+                sgmv_routed(y, v, B16, plan)
+            sbmm_2_4_routed(x_, DeltaW, metas, y, ss, idx32, index_offset=M, accumulate=True)
+            cur.wait_stream(side)
+            return y.to(x.dtype)
         cur.wait_stream(side)
         sgmv_routed(y, v, B16, plan)
     else:
