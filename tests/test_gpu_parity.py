@@ -45,6 +45,7 @@ def ops():
 @pytest.mark.parametrize("n,k,m,seed", [
     (1, 128, 256, 1), (3, 512, 256, 2), (16, 512, 256, 3), (17, 512, 256, 4), (64, 512, 384, 5),
     (100, 1024, 256, 6), (5, 192, 128, 7),            # k = 64 (mod 128): the partial last k step
+    (2, 64, 128, 13), (70, 64, 128, 14),              # the smallest layer: one partial k step, one column block
     (64, 256, 128, 8), (97, 320, 640, 9), (130, 192, 384, 10), (200, 512, 1408, 12),   # wide tiles, ragged ends
     (16, 4096, 4096, 1000),                           # BASELINE config 0
 ])
