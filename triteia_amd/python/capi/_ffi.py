@@ -93,3 +93,21 @@ def require_gpu(**tensors):
 def require_dtype(t, dtype, name):
     if t.dtype != dtype:
         raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
+
+
+_LOCK_WORKSPACES = {}
+
+
+def lock_workspace(numel: int, device) -> torch.Tensor:
+    """All-zero int32 tensor of at least `numel` elements for the lock `workspace` argument of
+    mul_2_4 / bmm_2_4 / sbmm_2_4.  The library checks its size and never reads or writes it, so
+    one tensor per device serves every call (the reference allocates and clears one per call)."""
+    dev = torch.device(device)
+    if dev.type != "cuda":      # the op itself rejects CPU tensors, with its own message
+        return torch.zeros(int(numel), dtype=torch.int32, device=dev)
+    key = dev.index if dev.index is not None else torch.cuda.current_device()
+    ws = _LOCK_WORKSPACES.get(key)
+    if ws is None or ws.numel() < numel:
+        ws = torch.zeros(max(int(numel), 4096), dtype=torch.int32, device=dev)
+        _LOCK_WORKSPACES[key] = ws
+    return ws
