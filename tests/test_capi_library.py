@@ -78,3 +78,16 @@ def test_python_wrappers_refuse_cpu_tensors():
     with pytest.raises(RuntimeError, match="GPU tensor"):
         matmul_4bit_2_4(torch.zeros(4, 512, dtype=torch.int32), x, torch.zeros(256, 8, dtype=torch.int16),
                         torch.ones(1, 256, dtype=torch.float16))
+
+
+def test_product_code_never_reaches_for_the_oracle():
+    """The CPU restatement is the checker: nothing in the package, its import alias, the C sources
+    or the header may import, read or mention it."""
+    import pathlib
+    root = pathlib.Path(__file__).resolve().parents[1]
+    offenders = []
+    for top in ("triteia_amd", "triteia", "include"):
+        for path in (root / top).rglob("*"):
+            if path.suffix in (".py", ".h", ".hip") and "oracle" in path.read_text(errors="replace"):
+                offenders.append(str(path.relative_to(root)))
+    assert not offenders, offenders

@@ -12,7 +12,7 @@ def _base(x, out_features, base_weight):
 
 
 def lora_forloop(weights_A, weights_B, x, indices, base_weight=None):
-    """torch oracle (lora.py:4-20). weights_A [M, k, r], weights_B [M, r, m]."""
+    """Per-token loop in torch (lora.py:4-20). weights_A [M, k, r], weights_B [M, r, m]."""
     y = _base(x, weights_B.shape[2], base_weight)
     if torch.all(indices == -1):
         return y
