@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the multi-model low-precision GEMM path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg0..cfg4] [--tokens T]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg0..cfg4|cfg3split] [--tokens T]
 
 A step is one pass of the hot path over one batch of synthetic input that is already
 resident in HBM: for the default workload (indexed sbmm, 64 tokens routed over 16 deltas of
@@ -37,7 +37,7 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
-    p.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
+    p.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg3split", "cfg4"])
     p.add_argument("--tokens", type=int, default=None, help="override the token count (cfg0/cfg2/cfg3/cfg4)")
     p.add_argument("--deltas", type=int, default=None, help="override the number of resident deltas (cfg4)")
     p.add_argument("--shape", default=None, help="K,M: override the weight shape (cfg0)")
@@ -75,6 +75,9 @@ class Problem:
             self.lora_b = (torch.randn((wl.n_lora, wl.lora_rank, wl.m), generator=g, device=dev) * 0.01).half()
             self.v = torch.zeros((wl.tokens, wl.lora_rank), dtype=torch.float16, device=dev)
             self.side = torch.cuda.Stream(device=dev)      # default priority
+            if wl.index_offset:
+                nb = self.lib.triteia_hip_sbmm_routed_workspace_bytes(wl.tokens, wl.n_lora)
+                self.ws_lora = torch.zeros((nb + 3) // 4, dtype=torch.int32, device=dev)
 
     def _chk(self, rc):
         if rc != 0:
@@ -85,7 +88,14 @@ class Problem:
 
     def plan(self):
         wl, P = self.wl, self.ffi.ptr
-        self._chk(self.lib.triteia_hip_route_plan(P(self.idx), 0, wl.n_deltas, wl.tokens, P(self.ws), self.ws_bytes, 0, self.stream()))
+        self._chk(self.lib.triteia_hip_route_plan(P(self.idx), wl.index_offset, wl.n_deltas, wl.tokens, P(self.ws), self.ws_bytes, 0,
+                                                  self.stream()))
+
+    def plan_lora(self):
+        """Split index space: the LoRA tokens (indices below index_offset) get a plan of their own."""
+        wl, P = self.wl, self.ffi.ptr
+        self._chk(self.lib.triteia_hip_route_plan(P(self.idx), 0, wl.n_lora, wl.tokens, P(self.ws_lora), self.ws_lora.numel() * 4, 0,
+                                                  self.stream()))
 
     def delta_kernel(self, i, accumulate=0):
         """Only the dominant kernel (on an existing plan for sbmm / ldmm)."""
@@ -102,6 +112,14 @@ class Problem:
             self._chk(self.lib.triteia_hip_sbmm_2_4_planned(P(self.x), P(q), P(me), P(self.out), P(s), P(self.ws), wl.n_deltas, wl.m,
                                                             wl.tokens, wl.k, accumulate, 0, st))
 
+    def delta_routed(self, i):
+        """Split index space: the routed delta multiply, added in place (indices below index_offset are not its rows)."""
+        wl, P = self.wl, self.ffi.ptr
+        q, me, s = self.weights[i % self.copies]
+        self._chk(self.lib.triteia_hip_sbmm_2_4_routed(P(self.x), P(q), P(me), P(self.out), P(s), P(self.idx), wl.index_offset,
+                                                       wl.n_deltas, wl.m, wl.tokens, wl.k, P(self.ws), self.ws_bytes, 1, 0,
+                                                       self.stream()))
+
     def step(self, i):
         """The whole hot path for one batch."""
         wl, P, torch = self.wl, self.ffi.ptr, self.torch
@@ -111,6 +129,25 @@ class Problem:
             q, me, s = self.weights[i % self.copies]
             self._chk(self.lib.triteia_hip_sbmm_2_4_routed(P(self.x), P(q), P(me), P(self.out), P(s), P(self.idx), 0, wl.n_deltas, wl.m,
                                                            wl.tokens, wl.k, P(self.ws), self.ws_bytes, 0, 0, self.stream()))
+        elif wl.index_offset:
+            # ldmm on a split index space, as triteia_amd.python.ops.ldmm runs it: LoRA plan, zero and shrink beside
+            # the base GEMM; then the expand (LoRA rows) beside the routed delta multiply (delta rows)
+            r = wl.lora_rank
+            cur, side = torch.cuda.current_stream(), self.side
+            q, me, s = self.weights[i % self.copies]
+            side.wait_stream(cur)
+            with torch.cuda.stream(side):
+                self.plan_lora()
+                self.v.zero_()
+                self._chk(self.lib.triteia_hip_sgmv_routed(P(self.v), r, P(self.x), wl.k, P(self.lora_a), wl.k * r, wl.n_lora,
+                                                           wl.k, r, 1.0, P(self.ws_lora), wl.tokens, 0, self.stream()))
+            torch.matmul(self.x, self.base[i % self.copies].t(), out=self.out)
+            side.wait_stream(cur)
+            with torch.cuda.stream(side):
+                self._chk(self.lib.triteia_hip_sgmv_routed(P(self.out), wl.m, P(self.v), r, P(self.lora_b), r * wl.m, wl.n_lora, r,
+                                                           wl.m, 1.0, P(self.ws_lora), wl.tokens, 0, self.stream()))
+            self.delta_routed(i)
+            cur.wait_stream(side)
         else:  # ldmm: dense base GEMM (library) + routed LoRA (SGMV) + routed delta, one routing plan for both
             r = wl.lora_rank
             cur = torch.cuda.current_stream()
@@ -144,8 +181,9 @@ def cpu_baseline(wl, torch, budget_s=20.0):
     from triteia_amd import workloads as W
     cores = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
-    used = sorted(set(int(i) for i in wl.indices if i >= 0)) if wl.indices is not None else list(range(wl.n_deltas))
-    counts = {d: (int((wl.indices == d).sum()) if wl.indices is not None else wl.tokens // wl.n_deltas) for d in used}
+    didx = wl.delta_indices()
+    used = sorted(set(int(i) for i in didx if i >= 0)) if didx is not None else list(range(wl.n_deltas))
+    counts = {d: (int((didx == d).sum()) if didx is not None else wl.tokens // wl.n_deltas) for d in used}
     x = W.random_activations(wl.tokens, wl.k, wl.seed + 1, "cpu").float()
     t_deq = t_mm = 0.0
     flops = 0.0
@@ -251,7 +289,7 @@ def main():
     ms_per_step = elapsed / a.steps * 1e3
     flops = wl.delta_flops()
     if wl.op == "ldmm":
-        flops += 2.0 * wl.tokens * wl.k * wl.m + 2.0 * wl.routed_tokens() * wl.lora_rank * (wl.k + wl.m)
+        flops += 2.0 * wl.tokens * wl.k * wl.m + 2.0 * wl.lora_tokens() * wl.lora_rank * (wl.k + wl.m)
     value = flops / (elapsed / a.steps) / 1e12
 
     # ---- dominant kernel alone: HIP events on the launch stream, batches of back-to-back launches
@@ -259,7 +297,7 @@ def main():
     # is routed inside the multiply kernel: the whole step is that one launch, and it is the kernel timed
     # here; otherwise the multiply runs on a routing plan)
     fused = wl.op == "sbmm" and ((wl.tokens <= 64 and wl.n_deltas <= 64) or (wl.tokens <= 256 and wl.n_deltas <= 32))
-    kernel_call = prob.step if fused else prob.delta_kernel
+    kernel_call = prob.step if fused else (prob.delta_routed if wl.index_offset else prob.delta_kernel)
     if wl.indices is not None and not fused:
         prob.plan()
     for i in range(5):

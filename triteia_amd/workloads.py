@@ -62,19 +62,36 @@ class Workload:
     lora_rank: int = 0
     n_lora: int = 0
     with_base: bool = False
+    index_offset: int = 0   # ldmm with the reference's split index space: [0, offset) = LoRA adapters, offset + d = delta d
 
     @property
     def delta_bytes(self):
         # int4 values of the kept half + 2 metadata bits per kept value + fp16 scales
         return self.k * self.m // 4 + self.k * self.m // 8 + 2 * self.m
 
+    def delta_indices(self):
+        """Per token: its delta, or -1 (no model, or a LoRA adapter of a split index space)."""
+        if self.indices is None:
+            return None
+        d = self.indices - self.index_offset
+        return np.where((self.indices >= self.index_offset) & (d < self.n_deltas), d, -1).astype(np.int32)
+
     def routed_tokens(self):
-        return self.tokens if self.indices is None else int((self.indices >= 0).sum())
+        return self.tokens if self.indices is None else int((self.delta_indices() >= 0).sum())
+
+    def lora_tokens(self):
+        """Tokens that take a LoRA adapter: all routed ones when LoRA shares the routing of the deltas."""
+        if self.n_lora == 0 or self.indices is None:
+            return 0
+        if self.index_offset == 0:
+            return self.routed_tokens()
+        return int(((self.indices >= 0) & (self.indices < self.index_offset)).sum())
 
     def distinct_deltas(self):
         if self.indices is None:
             return self.n_deltas
-        return int(len(np.unique(self.indices[self.indices >= 0])))
+        d = self.delta_indices()
+        return int(len(np.unique(d[d >= 0])))
 
     def delta_flops(self):
         """dense-equivalent 2*T_routed*k*m, the reference's convention (meta/benchmarks/bench_sbmm.py:17)."""
@@ -105,6 +122,15 @@ def config(name, tokens=None, shape=None):
         t = 256 if tokens is None else tokens
         return Workload(f"cfg3 ldmm 4096x11008, 32 deltas, {t} tokens Zipf(1.5) 10% -1, SGMV r=16 x 32", "ldmm", 4096, 11008,
                         32, t, 1003, indices=zipf_indices(t, 32, 1.5, 1003, 0.10), lora_rank=16, n_lora=32, with_base=True)
+    if name == "cfg3split":
+        # the same layer with the reference's ldmm index space (tests/ops/test_ldmm.py:34-64): a routed token
+        # takes either LoRA adapter i (index i) or delta i (index 32 + i), by a fair coin
+        t = 256 if tokens is None else tokens
+        idx = zipf_indices(t, 32, 1.5, 1003, 0.10)
+        coin = np.random.default_rng(2003).random(t) < 0.5
+        idx = np.where((idx >= 0) & coin, idx + 32, idx).astype(np.int32)
+        return Workload(f"cfg3split ldmm 4096x11008, {t} tokens Zipf(1.5) 10% -1, each to LoRA adapter i (r=16) or delta i of 32",
+                        "ldmm", 4096, 11008, 32, t, 1003, indices=idx, lora_rank=16, n_lora=32, with_base=True, index_offset=32)
     if name == "cfg4":
         t = 1024 if tokens is None else tokens
         return Workload(f"cfg4 sbmm 8192x28672, 64 deltas, {t} tokens Zipf(1.2)", "sbmm", 8192, 28672, 64, t, 1004,
