@@ -344,6 +344,22 @@ def main():
             "kernel_tflops": round(kflops, 2), "mfma_frac": round(kflops / MFMA_SPARSE_F16_TFLOPS, 4),
         }
 
+    # what this GPU delivers on a plain device-to-device copy (512 MiB read + 512 MiB written per launch), next to
+    # the nominal peak the fractions above are priced against
+    src = torch.empty(512 * 2 ** 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        dst.copy_(src)
+    e1.record()
+    e1.synchronize()
+    roofline["device_copy_gbs"] = round(2 * src.numel() * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9, 1)
+    del src, dst
+
     res = {
         "metric": "sbmm/ldmm dense-equivalent TFLOP/s at Llama-2-7B shapes (with % of HBM roofline)",
         "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
