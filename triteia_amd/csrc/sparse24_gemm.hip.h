@@ -181,7 +181,6 @@ struct TileCtx {
   // the parts in order.
   int raw_list[kRawParts];
   int raw_before[kRawParts + 1];
-  half8_t sv;               // scales of this thread's 8 output features (requested at start-up)
 #ifdef TRITEIA_HIP_TIMELINE
   long long ts[4];          // debug builds: entry, operands requested, K loop done, end
 #endif
@@ -247,6 +246,11 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
       load_w(ring[j], wave + j * KW);
     }
   }
+
+  // The scales of this thread's 8 output features, for the epilogue: requested here, behind the first
+  // weights, so that no wait for them can land ahead of a request (requested before the loop over
+  // passes they were waited for at the loop's entry: a full memory round trip before the first weights).
+  const half8_t sv = *reinterpret_cast<const half8_t*>(c.sc + (c.tid & 15) * 8);
 
   // Every lane always loads from a valid address, so that the number of loads per step is
   // fixed and the hardware load counter can be waited on exactly (the output columns of the
@@ -381,7 +385,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 #pragma unroll
         for (int i = 0; i < 4; i++) { v[i] += a0[i]; v[4 + i] += a1[i]; }
       }
-      const half8_t sv = c.sv;   // f0 is the same for every chunk of a thread: 64 * KW is a multiple of 16
+      // (sv: f0 is the same for every chunk of a thread, 64 * KW being a multiple of 16)
       _Float16* op = p.out + (long)row * p.out_stride + c.cb * 128 + f0;
       half8_t old = {0, 0, 0, 0, 0, 0, 0, 0};
       if (p.accumulate) old = *reinterpret_cast<const half8_t*>(op);
@@ -438,10 +442,11 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
     c.qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * c.r;
     c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.r >> 3)) * 16 + (c.r & 7);
     c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;
-    c.sv = *reinterpret_cast<const half8_t*>(c.sc + (c.tid & 15) * 8);
     // side-by-side deltas start their walks spread around the ring of steps (by the delta's index,
     // so that a result does not depend on where the weights happen to lie in memory)
-    c.rot = (int)(((long)delta * p.rot_spread) % c.n_steps);
+    // (32-bit arithmetic: a 64-bit remainder is a routine of some 150 instructions ahead of the first request;
+    // any value in [0, n_steps) is a valid start, so a wrapped product for a huge delta index does no harm)
+    c.rot = (int)(((unsigned)delta * (unsigned)p.rot_spread) % (unsigned)c.n_steps);
   };
 
   // group descriptor and live group count are fetched side by side (no dependent chain);
@@ -449,7 +454,7 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   int delta, start, count;
   bool alt_list = false;
   WPre pre[NPRE > 0 ? NPRE : 1];
-  if (p.raw_indices) {
+  if (EAGER || p.raw_indices) {   // (the eager build serves this form only: the others compile away)
     // Fused routing for small batches: every wavefront looks at all (<= 64) indices, one per
     // lane, and works out its delta and the rows routed to it -- a few dozen instructions
     // instead of a separate routing launch and a dependent descriptor read.
