@@ -75,8 +75,12 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   const int n_steps = (k_rows + 3) >> 2;
   const long qrow = p.m >> 1;
   const long mrow = p.m >> 2;
-  const uint4_t* qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cbc * 64 + 4 * r;
-  const uint4_t* mt_lane = p.meta + (long)delta * p.meta_stride + (long)cbc * 32 + (r >> 3) * 16 + (r & 7);
+  // operand addresses = a base that is the same for the whole wave (scalar registers) + a 32-bit byte
+  // offset per lane: two registers per lane fewer for each pointer that stays alive across the K loop
+  const uint4_t* qw_delta = p.qweight + (long)delta * p.qweight_stride;
+  const uint4_t* mt_delta = p.meta + (long)delta * p.meta_stride;
+  const uint32_t woff = (uint32_t)((q * qrow + (long)cbc * 64 + 4 * r) * 16);
+  const uint32_t moff = (uint32_t)((q * mrow + (long)cbc * 32 + (r >> 3) * 16 + (r & 7)) * 16);
 
   // token rows of the tile (slots past the end repeat the last row; their outputs are dropped)
   if (tid < kWideTokens) {
@@ -89,19 +93,28 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   // consecutive 16-byte chunks = 4 token rows; instruction ii of wave w covers rows
   // 16 ii + 4 w + lane/16.  Lane l fills chunk position l % 16 of its row, which holds the
   // row's chunk (l % 16) ^ (row % 16).
-  const _Float16* xsrc[4];
+  uint32_t xoff[4];   // byte offsets into x (the launcher sends activations of 4 GiB and more elsewhere)
 #pragma unroll
   for (int ii = 0; ii < 4; ii++) {
     const int row = 16 * ii + 4 * wave + (lane >> 4);
     const int chunk = (lane & 15) ^ (row & 15);
-    xsrc[ii] = p.x + (long)s_rows[row] * p.x_stride + chunk * 8;
+    xoff[ii] = (uint32_t)(((long)s_rows[row] * p.x_stride + chunk * 8) * 2);
   }
+  // Direct-to-LDS loads and the waits for them are written as inline assembly: the compiler
+  // counts a direct-to-LDS load as an LDS write, which the release fence of every barrier and
+  // the first LDS read behind it must complete, i.e. it drains every outstanding request (the
+  // weights requested a moment ago included) once per K step.  The LDS address of a request is
+  // M0 + 16 * lane.
+  const uint32_t lds_x_wave = (uint32_t)(uintptr_t)&xs[0][4 * wave][0];
   auto issue_x = [&](int st) {
     const int stc = min(st, n_steps - 1);   // past the end: refetch the last tile (never read)
     const int stage = st & (kWideStages - 1);
 #pragma unroll
-    for (int ii = 0; ii < 4; ii++)
-      __builtin_amdgcn_global_load_lds(xsrc[ii] + stc * 128, &xs[stage][16 * ii + 4 * wave][0], 16, 0, 0);
+    for (int ii = 0; ii < 4; ii++) {
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_x_wave + (stage * kWideTokens + 16 * ii) * 256);
+      const _Float16* base = p.x + stc * 128;
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(xoff[ii]), "s"(base), "s"(dst) : "memory");
+    }
   };
 
   struct WFrag {
@@ -109,14 +122,13 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
     uint4_t mt[2];
   };
   auto load_w = [&](WFrag& f, int st) {
-    const int tr0 = (st < n_steps ? st : 0) << 2;
-    const int tr = min(tr0 + q, k_rows - 1);   // rows past the end of K meet zero activations
-    const uint4_t* wp = qw_lane + (long)tr * qrow;
-    const uint4_t* mp = mt_lane + (long)tr * mrow;
+    const long tr0 = (st < n_steps ? st : 0) << 2;   // past the end: any valid rows (never used); k % 128 == 0, so
+    const char* wb = reinterpret_cast<const char*>(qw_delta + tr0 * qrow);   // rows tr0 .. tr0 + 3 always exist
+    const char* mb = reinterpret_cast<const char*>(mt_delta + tr0 * mrow);
 #pragma unroll
-    for (int a = 0; a < 4; a++) f.wq[a] = wp[a];
-    f.mt[0] = mp[0];
-    f.mt[1] = mp[8];
+    for (int a = 0; a < 4; a++) f.wq[a] = *reinterpret_cast<const uint4_t*>(wb + woff + 16 * a);
+    f.mt[0] = *reinterpret_cast<const uint4_t*>(mb + moff);
+    f.mt[1] = *reinterpret_cast<const uint4_t*>(mb + moff + 128);
   };
 
   float4_t acc[8][NT];
@@ -180,30 +192,33 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
     }
   };
 
-  // pipeline: weights DEPTH steps ahead in registers; activation tiles 3 steps ahead in the
-  // LDS ring.  At the top of step st this wave waits until its own direct loads of tile st
-  // have landed (everything it issued since then is allowed to stay in flight: 4 loads for each
-  // of tiles st+1 and st+2 at least), then the barrier makes all four waves' parts visible
-  // and also says that tile st-1 has been read by everyone, so its stage can be refilled.
+  // pipeline: weights DEPTH steps ahead in registers (requests the compiler tracks), activation tiles
+  // 3 steps ahead in the LDS ring (requests it does not see).  Requests complete in order, and every
+  // step issues its activation tile first and its weights last, so the compiler's wait for the weights of
+  // step st ("all but the newest 6 (DEPTH - 1) requests") is exact for DEPTH = 2: the weights of step
+  // st + 1 stay in flight across the step.  The hand-written wait at the top of a step says that this
+  // wave's part of tile st has landed: behind it in the queue are at most the tiles st+1, st+2 (8
+  // requests) and DEPTH sets of weights (6 each); the barrier then makes all four waves' parts visible and
+  // also says that tile st-1 has been read by everyone, so its stage can be refilled.
   WFrag ring[DEPTH];
-#pragma unroll
-  for (int j = 0; j < DEPTH; j++) load_w(ring[j], j);
   issue_x(0);
   issue_x(1);
   issue_x(2);
+#pragma unroll
+  for (int j = 0; j < DEPTH; j++) load_w(ring[j], j);
   constexpr int TURN = DEPTH > 4 ? DEPTH : 4;   // whole ring turns of both rings (DEPTH divides 4)
   for (int s0 = 0; s0 < n_steps; s0 += TURN) {
 #pragma unroll
     for (int j = 0; j < TURN; j++) {
       const int st = s0 + j;
-      __builtin_amdgcn_s_waitcnt(0x0F70 | 8);   // vmcnt(8), nothing else
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(8 + 6 * DEPTH) : "memory");
       lds_barrier();
-      issue_x(st + 3);
       if (st < n_steps && active) compute_step(ring[j % DEPTH], j & (kWideStages - 1));
+      issue_x(st + 3);
       load_w(ring[j % DEPTH], st + DEPTH);
     }
   }
-  __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): no direct load may outlive the block's LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive the block's LDS
 
   if (!active) return;
   // epilogue: lane (n = r, qq = q) holds features 32q + 8j + c of token n for every 16-token tile

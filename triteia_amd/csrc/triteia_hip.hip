@@ -221,7 +221,7 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   a.delta_step = delta_step;
   const long cgs = (a.m / 128 + 3) / 4;
   int done = 0;
-  // (the 128-token kernel addresses activations with 32-bit byte offsets)
+  // (the wide kernels address activations with 32-bit byte offsets)
   const bool x_below_4g = ((long)(n_groups - 1) * stride + tokens) * a.x_stride * 2 < (1L << 32);
   // (the 128-token kernel pays from k = 8192 on: 2-3 % faster than the 64-token kernel at 8192 x 8192 and
   // 8192 x 28672, 4-8 % slower at 4096 x 4096 and 4096 x 11008, whose K loops are too short for its pipeline)
@@ -235,7 +235,7 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
     done = t;
   }
   int rest = tokens - done;
-  if (rest > 0 && wide_enabled() && a.k % 128 == 0 &&
+  if (rest > 0 && wide_enabled() && a.k % 128 == 0 && x_below_4g &&
       (done > 0 ? rest >= kPlanWideMinRest
                 : (long)n_groups * (rest / kWideTokens) * cgs >= env_int("TRITEIA_HIP_WIDE_MIN_UNITS", kWideMinUnits))) {
     int t = rest / kWideTokens * kWideTokens;
@@ -393,7 +393,9 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     // The wide kernel needs whole 128-deep K steps, and a batch that could not reach the bar
     // even with most of its tokens in wide tiles (one per 48 tokens) is not worth the empty
     // launch: then the bar is out of reach on the device too and every tile list is the narrow-only one.
-    wide_launch = prob_k % 128 == 0 && (long)(prob_n / 48 + 1) * a.wide_gate >= a.wide_min_units;
+    // (and it addresses activations with 32-bit byte offsets)
+    wide_launch = prob_k % 128 == 0 && (long)prob_n * prob_k * 2 < (1L << 32) &&
+                  (long)(prob_n / 48 + 1) * a.wide_gate >= a.wide_min_units;
     if (!wide_launch) a.wide_min_units = 0x7fffffff;
   }
   // The plan's tiles are cut without knowledge of the layer.  Where they make a launch of very few
