@@ -155,11 +155,13 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
     // Per k-half u and per half of the 8 columns: dequantise 4 weight fragments, then run them
     // against the four 16-token B fragments.  B fragments are read one ahead of the MFMAs that
     // use them, so that the LDS latency hides behind 4 MFMAs instead of stalling in front of them.
-    half16_t b_nxt = read_b(stage, 0, 0);
+    half16_t b_nxt;
+    if (DEPTH < 2) b_nxt = read_b(stage, 0, 0);
 #pragma unroll
     for (int u = 0; u < 2; u++) {
 #pragma unroll
       for (int b2 = 0; b2 < 2; b2++) {
+        if (DEPTH >= 2) __builtin_amdgcn_sched_barrier(0);   // (keeps the scheduler from pulling later fragments ahead: registers)
         half8_t A[4];
 #pragma unroll
         for (int w = 0; w < 4; w++) {
@@ -174,10 +176,15 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
         }
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
-          const half16_t b = b_nxt;
-          if (nt + 1 < NT) b_nxt = read_b(stage, nt + 1, u);
-          else if (b2 == 0) b_nxt = read_b(stage, 0, u);
-          else if (u == 0) b_nxt = read_b(stage, 0, 1);
+          half16_t b;
+          if (DEPTH < 2) {
+            b = b_nxt;
+            if (nt + 1 < NT) b_nxt = read_b(stage, nt + 1, u);
+            else if (b2 == 0) b_nxt = read_b(stage, 0, u);
+            else if (u == 0) b_nxt = read_b(stage, 0, 1);
+          } else {
+            b = read_b(stage, nt, u);   // (two steps of weights in flight leave no registers for a fragment ahead)
+          }
 #pragma unroll
           for (int w = 0; w < 4; w++) {
             const int cc = 4 * b2 + w;

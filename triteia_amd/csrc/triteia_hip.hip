@@ -205,10 +205,13 @@ int launch_wide128(const Sparse24Args& a, hipStream_t st) {
 }
 
 // The wide kernels pay off when there are enough tiles to occupy the GPU; below that the
-// narrow kernel's smaller units win.  TRITEIA_HIP_WIDE=0 disables both, TRITEIA_HIP_WIDE128=0
-// the 128-token one; TRITEIA_HIP_WIDE_MIN_UNITS / TRITEIA_HIP_WIDE128_MIN_UNITS move the thresholds.
+// narrow kernel's smaller units win.  TRITEIA_HIP_WIDE=0 disables both; the 128-token one is off unless
+// TRITEIA_HIP_WIDE128=1 (since the 64-token kernel's requests stay in flight across its barriers it is
+// as fast or faster on every shape measured: 4096 tokens on 8192 x 8192 279-296 us against 286-301 us, on
+// 8192 x 28672 970 us both, 1024 tokens there 258 against 270 us);
+// TRITEIA_HIP_WIDE_MIN_UNITS / TRITEIA_HIP_WIDE128_MIN_UNITS move the thresholds.
 bool wide_enabled() { return env_int("TRITEIA_HIP_WIDE", 1) != 0; }
-bool wide128_enabled() { return wide_enabled() && env_int("TRITEIA_HIP_WIDE128", 1) != 0; }
+bool wide128_enabled() { return wide_enabled() && env_int("TRITEIA_HIP_WIDE128", 0) != 0; }
 constexpr long kWideMinUnits = 160;   // 4096 x 4096: 1024 tokens (128 tiles) 54.9 us wide against 46.5 us narrow, 1536 tokens (192) 60.8 against 71.1
 constexpr long kWide128MinUnits = 192;
 
