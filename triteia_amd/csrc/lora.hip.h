@@ -15,7 +15,7 @@
 #include <stdint.h>
 
 #ifndef TRITEIA_SHRINK_UNROLL
-#define TRITEIA_SHRINK_UNROLL 8
+#define TRITEIA_SHRINK_UNROLL 4
 #endif
 
 namespace triteia_hip {
@@ -24,6 +24,14 @@ typedef _Float16 lhalf8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 lhalf2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kLoraMaxNarrow = 128;
+
+// Load through a pointer that is known to point into global memory.  (An adapter pointer read from the
+// caller's pointer table is a generic pointer to the compiler: its loads become flat loads, which count
+// against the LDS / scalar counter as well and are waited for more conservatively.)
+template <class T>
+__device__ __forceinline__ T load_global(const T* p) {
+  return *(const __attribute__((address_space(1))) T*)(uintptr_t)p;
+}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -135,6 +143,23 @@ __device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* 
 
 __device__ __forceinline__ int sgmv_row(const SgmvArgs& a, int i) { return a.perm ? a.perm[i] : i; }
 
+// The rows of R consecutive list positions (positions past the end of the group repeat `first`).  The list
+// entries are requested together and without a branch around the loads (a load under a branch is waited for
+// where the branches join: one memory round trip per row); without a list the same loads read the head of
+// the activations, which is always there, and their values are dropped.
+template <int R>
+__device__ __forceinline__ void sgmv_rows(const SgmvArgs& a, int first, int n_left, int (&rows)[R]) {
+  const int* list = a.perm ? a.perm : reinterpret_cast<const int*>(a.x);
+  int pos[R], listed[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    pos[r] = first + (r < n_left ? r : 0);
+    listed[r] = list[a.perm ? pos[r] : 0];
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++) rows[r] = a.perm ? listed[r] : pos[r];
+}
+
 // wide -> narrow (d_out <= DOUT <= 128): grid (n_groups, row slots), block 256; a block takes
 // R token rows of its group at a time and walks all of d_in once for them.  With CB = d_out / 8
 // column blocks, thread (kp, cb) = (tid / CB, tid % CB) reads the 16-byte pieces [k][cb*8 .. +8] of
@@ -161,28 +186,43 @@ __global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgs a) {
   for (int r0 = blockIdx.y * R; r0 < g.count; r0 += gridDim.y * R) {
     int rows[R];
     const _Float16* xr[R];
+    sgmv_rows<R>(a, g.start + r0, g.count - r0, rows);
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      rows[r] = sgmv_row(a, g.start + (r0 + r < g.count ? r0 + r : r0));
-      xr[r] = a.x + (long)rows[r] * a.x_stride;
-    }
+    for (int r = 0; r < R; r++) xr[r] = a.x + (long)rows[r] * a.x_stride;
     float acc[R][8];
 #pragma unroll
     for (int r = 0; r < R; r++)
 #pragma unroll
       for (int j = 0; j < 8; j++) acc[r][j] = 0.f;
     if (worker) {
+      // U sweeps at a time: their loads are all requested before the first is used (no branch between them:
+      // a sweep past the end of K re-reads the batch's first rows and meets zero activations), so a thread
+      // has U times the requests in flight and a U-th of the round trips in sequence.  Sums are taken in
+      // the order of k, as without the batching.
+      constexpr int U = TRITEIA_SHRINK_UNROLL;
       const _Float16* wp = g.w + cb * 8;
-#pragma unroll TRITEIA_SHRINK_UNROLL
-      for (int k = 2 * kp; k < a.d_in; k += 2 * KP) {
-        const lhalf8_t w0 = *reinterpret_cast<const lhalf8_t*>(wp + (long)k * dn);
-        const lhalf8_t w1 = *reinterpret_cast<const lhalf8_t*>(wp + (long)(k + 1) * dn);
+      const int kstep = 2 * KP;
+      for (int k0 = 2 * kp; k0 < a.d_in; k0 += U * kstep) {
+        lhalf8_t w0[U], w1[U];
+        lhalf2_t xv[U][R];
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-          const lhalf2_t xv = *reinterpret_cast<const lhalf2_t*>(xr[r] + k);
-          const float x0 = (float)xv[0], x1 = (float)xv[1];
+        for (int u = 0; u < U; u++) {
+          const int k = k0 + u * kstep;
+          const int kc = k < a.d_in ? k : k0;
+          w0[u] = load_global(reinterpret_cast<const lhalf8_t*>(wp + (long)kc * dn));
+          w1[u] = load_global(reinterpret_cast<const lhalf8_t*>(wp + (long)(kc + 1) * dn));
 #pragma unroll
-          for (int j = 0; j < 8; j++) acc[r][j] += x0 * (float)w0[j] + x1 * (float)w1[j];
+          for (int r = 0; r < R; r++) xv[u][r] = *reinterpret_cast<const lhalf2_t*>(xr[r] + kc);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          const bool live = k0 + u * kstep < a.d_in;
+#pragma unroll
+          for (int r = 0; r < R; r++) {
+            const float x0 = live ? (float)xv[u][r][0] : 0.f, x1 = live ? (float)xv[u][r][1] : 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[r][j] += x0 * (float)w0[u][j] + x1 * (float)w1[u][j];
+          }
         }
       }
     }
@@ -249,26 +289,37 @@ __global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgs a) 
   if (!sgmv_group(a, blockIdx.x, &g)) return;
   const int j0 = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (j0 >= a.d_out) return;
+  int r0 = blockIdx.z * R;
+  if (r0 >= g.count) return;
+  // Order of the requests: the first rows' list entries, then the weight patch, then (once the rows are
+  // known) their activations and old outputs; nothing is waited for before all of these are on their way.
+  int rows[R];
+  sgmv_rows<R>(a, g.start + r0, g.count - r0, rows);
   lhalf8_t w[DIN];
 #pragma unroll
-  for (int i = 0; i < DIN; i++) {
-    if (i < a.d_in) w[i] = *reinterpret_cast<const lhalf8_t*>(g.w + (long)i * a.d_out + j0);
-    else w[i] = lhalf8_t{0, 0, 0, 0, 0, 0, 0, 0};
-  }
-  for (int r0 = blockIdx.z * R; r0 < g.count; r0 += gridDim.z * R) {
+  for (int i = 0; i < DIN; i++)   // (no branch around a load: rows past d_in re-read the last one and are zeroed below)
+    w[i] = load_global(reinterpret_cast<const lhalf8_t*>(g.w + (long)(i < a.d_in ? i : a.d_in - 1) * a.d_out + j0));
+  bool patch_ready = false;
+  for (;;) {
     lhalf8_t xv[R][DIN / 8], old[R];
     _Float16* yp[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      const int row = sgmv_row(a, g.start + (r0 + r < g.count ? r0 + r : r0));
-      const _Float16* xr = a.x + (long)row * a.x_stride;
-      yp[r] = a.y + (long)row * a.y_stride + j0;
+      const _Float16* xr = a.x + (long)rows[r] * a.x_stride;
+      yp[r] = a.y + (long)rows[r] * a.y_stride + j0;
 #pragma unroll
       for (int i0 = 0; i0 < DIN / 8; i0++)
-        xv[r][i0] = i0 * 8 < a.d_in ? *reinterpret_cast<const lhalf8_t*>(xr + i0 * 8)   // same address in every lane
-                                    : lhalf8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        xv[r][i0] = *reinterpret_cast<const lhalf8_t*>(xr + (i0 * 8 < a.d_in ? i0 * 8 : 0));   // same address in every lane
       old[r] = *reinterpret_cast<const lhalf8_t*>(yp[r]);
     }
+    __builtin_amdgcn_sched_barrier(0);   // every request above is issued before the first result is touched
+    if (!patch_ready) {
+#pragma unroll
+      for (int i = 0; i < DIN; i++)
+        if (i >= a.d_in) w[i] = lhalf8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      patch_ready = true;
+    }
+    const int n_left = g.count - r0;
 #pragma unroll
     for (int r = 0; r < R; r++) {
       float acc[8];
@@ -281,8 +332,11 @@ __global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgs a) 
       lhalf8_t o;
 #pragma unroll
       for (int e = 0; e < 8; e++) o[e] = (_Float16)((float)old[r][e] + acc[e] * a.scale);
-      if (r == 0 || r0 + r < g.count) *reinterpret_cast<lhalf8_t*>(yp[r]) = o;
+      if (r == 0 || r < n_left) *reinterpret_cast<lhalf8_t*>(yp[r]) = o;
     }
+    r0 += gridDim.z * R;
+    if (r0 >= g.count) break;
+    sgmv_rows<R>(a, g.start + r0, g.count - r0, rows);
   }
 }
 
