@@ -393,6 +393,52 @@ def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, 
         assert torch.equal(o, outs[0])
 
 
+@pytest.mark.parametrize("T,N,k,m,seed,wide_bar", [
+    (100, 7, 256, 640, 101, "200"),        # ragged tiles, a partial last group of column blocks
+    (300, 40, 384, 1408, 102, "200"),      # most deltas with a handful of tokens
+    (90, 3, 128, 128, 103, "200"),         # one K step, one column block (three of four wavefronts idle)
+    (600, 40, 256, 512, 104, "1"),         # plan with wide tiles: this kernel takes the narrow-only list of the plan,
+    (600, 40, 256, 512, 105, "100000"),    # whatever the bar for the wide tiles says
+])
+def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, seed, wide_bar):
+    """A plan's 32-token tiles on a wide layer run on the 32-token build of the wide kernel (forced here
+    onto small layers).  Against the oracle within the bar; against the K-split kernel within rounding;
+    untouched rows stay untouched; accumulation in place."""
+    say(f"32-token wide kernel T={T} N={N} k={k} m={m} seed={seed} wide_bar={wide_bar}")
+    from triteia_amd.python.capi import sbmm_2_4_routed
+    monkeypatch.setenv("TRITEIA_HIP_FUSED_ROUTE", "0")
+    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", wide_bar)
+    qw, meta, s = make_deltas(N, k, m, seed)
+    x = activations(T, k, seed + 1)
+    idx = np.random.default_rng(seed + 2).integers(-1, N, size=T).astype(np.int32)
+    if wide_bar != "200":
+        idx[: T // 3] = 1                                      # a hot delta: several wide tiles
+    ref = orc.sbmm_4bit_2_4(qw, x, meta, s, idx)
+    gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
+    outs = {}
+    for mid in ("1", "0"):
+        monkeypatch.setenv("TRITEIA_HIP_MID", mid)
+        monkeypatch.setenv("TRITEIA_HIP_MID_MIN_UNITS", "1")
+        out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
+        sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
+        torch.cuda.synchronize()
+        outs[mid] = out
+    none = torch.from_numpy(idx < 0).to(DEV)
+    assert bool((outs["1"][none] == -3.0).all())
+    got = torch.where(none[:, None], torch.zeros_like(outs["1"]), outs["1"])
+    check_close(got, ref, what="32-token wide kernel")
+    assert not torch.equal(outs["1"], outs["0"]) or k <= 128, "the knob did not change the kernel"
+    assert float((outs["1"].float() - outs["0"].float()).norm()) <= 1e-3 * float(outs["0"].float().norm())
+    # accumulate in place on top of a base
+    monkeypatch.setenv("TRITEIA_HIP_MID", "1")
+    base = torch.from_numpy(activations(T, m, seed + 3)).to(DEV)
+    acc = base.clone()
+    sbmm_2_4_routed(gx, gq, gm, acc, gs, gi, accumulate=True)
+    torch.cuda.synchronize()
+    assert torch.equal(acc[none], base[none])
+    check_close(acc.float() - base.float(), ref, tol=4e-3, what="32-token wide kernel, accumulate")
+
+
 def test_empty_and_degenerate_inputs(ops):
     """Zero tokens, zero deltas, zero adapters, a batch in which nothing is routed: every op returns the
     shape it should and touches nothing else."""

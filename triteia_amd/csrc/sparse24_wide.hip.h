@@ -25,11 +25,12 @@ namespace triteia_hip {
 constexpr int kWideTokens = 64;
 constexpr int kWideStages = 4;        // activation tiles in flight (LDS ring)
 
-template <int DEPTH>
+// TOK: token rows of a tile (64, or 32 for the narrow tiles of a routing plan)
+template <int DEPTH, int TOK = kWideTokens>
 __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Args p) {
-  constexpr int NT = kWideTokens / 16;
-  __shared__ __attribute__((aligned(1024))) _Float16 xs[kWideStages][kWideTokens][128];
-  __shared__ int s_rows[kWideTokens];
+  constexpr int NT = TOK / 16;
+  __shared__ __attribute__((aligned(1024))) _Float16 xs[kWideStages][TOK][128];
+  __shared__ int s_rows[TOK];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -49,23 +50,33 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   const int cg = p.xcd_swizzle ? (i & 7) * (cg_pad >> 3) + (i >> 3) : i;
   if (cg >= cgs) return;
   int delta, start, count;
+  bool alt_list = false;
   if (p.tiles) {
-    const int4 d = p.tiles[grp];
+    int4 d = p.tiles[grp];
+    if (TOK == 32 && p.tiles_alt) {
+      // the 32-token build stands in for the narrow kernel on a plan's narrow tiles: like that kernel it takes
+      // the narrow-only list when the plan's wide tiles do not fill the chip (both candidates are requested together)
+      const int4 d_alt = p.tiles_alt[grp];
+      if ((long)p.n_groups_dev[4] * p.wide_gate < p.wide_min_units) {
+        d = d_alt;
+        alt_list = true;
+      }
+    }
     delta = d.x;
     start = d.y;
     count = d.z;
   } else {
-    const int chunks = (p.uniform_count + kWideTokens - 1) / kWideTokens;
+    const int chunks = (p.uniform_count + TOK - 1) / TOK;
     const int gi = grp / chunks, tc = grp - gi * chunks;
     delta = gi * p.delta_step;
-    start = gi * p.uniform_stride + p.uniform_first + tc * kWideTokens;
-    count = min(kWideTokens, p.uniform_count - tc * kWideTokens);
+    start = gi * p.uniform_stride + p.uniform_first + tc * TOK;
+    count = min(TOK, p.uniform_count - tc * TOK);
   }
-  const int n_groups = p.n_groups_dev ? *p.n_groups_dev : p.n_groups;
-  if (p.wide_min_units && (long)n_groups * p.wide_gate < p.wide_min_units) return;   // the narrow kernel has taken these tokens
+  const int n_groups = p.n_groups_dev ? p.n_groups_dev[alt_list ? 5 : 0] : p.n_groups;
+  if (TOK != 32 && p.wide_min_units && (long)n_groups * p.wide_gate < p.wide_min_units) return;   // the narrow kernel has taken these tokens
   if (grp >= n_groups) return;
   if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
-  const int cnt = min(count, kWideTokens);
+  const int cnt = min(count, TOK);
 
   const int cb = 4 * cg + wave;
   const bool active = cb < col_blocks;          // the last group of a matrix may be partial
@@ -83,7 +94,7 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   const uint32_t moff = (uint32_t)((q * mrow + (long)cbc * 32 + (r >> 3) * 16 + (r & 7)) * 16);
 
   // token rows of the tile (slots past the end repeat the last row; their outputs are dropped)
-  if (tid < kWideTokens) {
+  if (tid < TOK) {
     const int slot = min(tid, cnt - 1);
     s_rows[tid] = p.perm ? p.perm[start + slot] : start + slot;
   }
@@ -93,9 +104,9 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   // consecutive 16-byte chunks = 4 token rows; instruction ii of wave w covers rows
   // 16 ii + 4 w + lane/16.  Lane l fills chunk position l % 16 of its row, which holds the
   // row's chunk (l % 16) ^ (row % 16).
-  uint32_t xoff[4];   // byte offsets into x (the launcher sends activations of 4 GiB and more elsewhere)
+  uint32_t xoff[NT];   // byte offsets into x (the launcher sends activations of 4 GiB and more elsewhere)
 #pragma unroll
-  for (int ii = 0; ii < 4; ii++) {
+  for (int ii = 0; ii < NT; ii++) {
     const int row = 16 * ii + 4 * wave + (lane >> 4);
     const int chunk = (lane & 15) ^ (row & 15);
     xoff[ii] = (uint32_t)(((long)s_rows[row] * p.x_stride + chunk * 8) * 2);
@@ -110,8 +121,8 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
     const int stc = min(st, n_steps - 1);   // past the end: refetch the last tile (never read)
     const int stage = st & (kWideStages - 1);
 #pragma unroll
-    for (int ii = 0; ii < 4; ii++) {
-      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_x_wave + (stage * kWideTokens + 16 * ii) * 256);
+    for (int ii = 0; ii < NT; ii++) {
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_x_wave + (stage * TOK + 16 * ii) * 256);
       const _Float16* base = p.x + stc * 128;
       asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(xoff[ii]), "s"(base), "s"(dst) : "memory");
     }
@@ -204,8 +215,8 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   // step issues its activation tile first and its weights last, so the compiler's wait for the weights of
   // step st ("all but the newest 6 (DEPTH - 1) requests") is exact for DEPTH = 2: the weights of step
   // st + 1 stay in flight across the step.  The hand-written wait at the top of a step says that this
-  // wave's part of tile st has landed: behind it in the queue are at most the tiles st+1, st+2 (8
-  // requests) and DEPTH sets of weights (6 each); the barrier then makes all four waves' parts visible and
+  // wave's part of tile st has landed: behind it in the queue are at most the tiles st+1, st+2 (NT
+  // requests each) and DEPTH sets of weights (6 each); the barrier then makes all four waves' parts visible and
   // also says that tile st-1 has been read by everyone, so its stage can be refilled.
   WFrag ring[DEPTH];
   issue_x(0);
@@ -218,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
 #pragma unroll
     for (int j = 0; j < TURN; j++) {
       const int st = s0 + j;
-      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(8 + 6 * DEPTH) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NT + 6 * DEPTH) : "memory");
       lds_barrier();
       if (st < n_steps && active) compute_step(ring[j % DEPTH], j & (kWideStages - 1));
       issue_x(st + 3);

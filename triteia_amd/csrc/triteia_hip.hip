@@ -342,6 +342,19 @@ int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas) {
 // layer >= kPlanWideMinUnits); otherwise re-reading a hot delta's weights from cache in narrow
 // tiles is cheaper than a second, poorly filled launch, and the wide launch returns at once.
 constexpr int kPlanWideMinUnits = 200;
+// A plan's 32-token tiles on a wide layer go to the 32-token build of the wide kernel (four column blocks of a
+// workgroup share each activation tile through LDS, every wavefront walks all of K) instead of the K-split narrow
+// kernel, whose column-block workgroups each fetch the tile's activations again: 5-10 % faster once there are
+// about 450 (tile, 512-column group) units (cfg3 at 128 / 256 / 512 tokens 66.6 -> 62.7, 97 -> 88, 133 -> 126.5 us;
+// 8 deltas of 8192 x 28672 with 96 tokens 142 -> 128.5 us), slower below (16 deltas of 4096 x 4096 with 256 tokens
+// 24.9 -> 42.4 us).  The host only has the upper bound on the tiles; 600 on that bound separates the measured cases.
+constexpr int kMidMinUnits = 600;
+static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
+  if (!env_int("TRITEIA_HIP_MID", 1) || triteia_hip_plan_tile_tokens(prob_n, n_deltas) != 32) return false;
+  if (prob_k % 128 != 0 || (long)prob_n * prob_k * 2 >= (1L << 32)) return false;   // whole K steps, 32-bit activation offsets
+  const long tiles = (n_deltas < prob_n ? n_deltas : prob_n) + prob_n / 32;
+  return tiles * ((prob_m / 128 + 3) / 4) >= env_int("TRITEIA_HIP_MID_MIN_UNITS", kMidMinUnits);
+}
 constexpr int kFusedMaxTokens = 64 * kRawParts;   // kRawParts tokens per lane of a wavefront
 static int plan_has_wide(int prob_n, int n_deltas) {
   const long groups = n_deltas < prob_n ? n_deltas : prob_n;
@@ -388,6 +401,7 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
   a.n_groups = plan_max_tiles(prob_n, n_deltas, tile);
   a.accumulate = accumulate;
   const bool wide = plan_has_wide(prob_n, n_deltas);
+  const bool mid = mid_tiles(prob_n, n_deltas, prob_m, prob_k);
   bool wide_launch = false;
   if (wide) {
     a.tiles_alt = reinterpret_cast<const int4*>(ws + L.all);
@@ -397,7 +411,9 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     // even with most of its tokens in wide tiles (one per 48 tokens) is not worth the empty
     // launch: then the bar is out of reach on the device too and every tile list is the narrow-only one.
     // (and it addresses activations with 32-bit byte offsets)
-    wide_launch = prob_k % 128 == 0 && (long)prob_n * prob_k * 2 < (1L << 32) &&
+    // Nor is it where the 32-token wide kernel takes the plan's tiles: that kernel on the narrow-only list is
+    // as fast or faster than a split between the two (cfg4 at 512 / 768 tokens 955 -> 913 / 1075 -> 1032 us).
+    wide_launch = !mid && prob_k % 128 == 0 && (long)prob_n * prob_k * 2 < (1L << 32) &&
                   (long)(prob_n / 48 + 1) * a.wide_gate >= a.wide_min_units;
     if (!wide_launch) a.wide_min_units = 0x7fffffff;
   }
@@ -415,6 +431,13 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     const int forced = env_int("TRITEIA_HIP_PASS_NT", 0);
     if ((forced == 1 || forced == 2 || forced == 4) && 16 * forced <= tile) pass_nt = forced;
   }
+  if (mid) {
+    const long cgs = (a.m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
+    if ((long)a.n_groups * cg_pad > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units");
+    hipLaunchKernelGGL((sparse24_wide_kernel<1, 32>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), a);
+    if (int e = check_launch("sparse24_wide_kernel<32>")) return e;
+  } else
   if (int e = launch_sparse24(a, pass_nt, tile / (16 * pass_nt), static_cast<hipStream_t>(stream))) return e;
   if (wide_launch) {
     a.tiles = reinterpret_cast<const int4*>(ws + L.wide);
@@ -436,8 +459,13 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null tensor pointer");
   // (above 64 tokens only for at most 32 deltas: with 64 deltas of 8192 x 28672 under a skewed routing the
   // workgroups of the deltas without tokens make this form 1-2 % slower than a plan, which lists none)
+  // (and from 128 tokens on, a batch whose deltas' weights are not requested ahead of the routing is better
+  // off with a plan where the plan's tiles go to the 32-token wide kernel: 32 deltas of 4096 x 11008,
+  // 128 / 256 tokens: 69 -> 65.5 / 96 -> 89.5 us including the plan)
+  const bool eager_ok = n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && env_int("TRITEIA_HIP_EAGER", 1);
   if (prob_n <= env_int("TRITEIA_HIP_FUSED_MAX_TOKENS", kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
-      n_deltas <= (prob_n > 64 ? 32 : 64) && env_int("TRITEIA_HIP_FUSED_ROUTE", 1)) {
+      n_deltas <= (prob_n > 64 ? 32 : 64) && env_int("TRITEIA_HIP_FUSED_ROUTE", 1) &&
+      !(prob_n >= 128 && !eager_ok && mid_tiles(prob_n, n_deltas, prob_m, prob_k))) {
     // small batch: the multiply kernel routes by itself, no plan, no workspace traffic
     if (!token_indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null indices");
     DeviceGuard g(dev);
@@ -456,7 +484,7 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
     // first.  Only for at most 16 deltas: under a skewed routing larger sets leave many deltas
     // without a token (Zipf(1.5) over 32: 14 in use at 64 tokens, and the prefetched steps of the
     // other 18 make the launch 10 % slower than routing first).
-    if (n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && env_int("TRITEIA_HIP_EAGER", 1)) {
+    if (eager_ok) {
       a.raw_static = 1;
       a.n_groups = n_deltas;
     }
