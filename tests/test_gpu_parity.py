@@ -399,6 +399,8 @@ def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, 
     (90, 3, 128, 128, 103, "200"),         # one K step, one column block (three of four wavefronts idle)
     (600, 40, 256, 512, 104, "1"),         # plan with wide tiles: this kernel takes the narrow-only list of the plan,
     (600, 40, 256, 512, 105, "100000"),    # whatever the bar for the wide tiles says
+    (600, 6, 256, 640, 106, "1"),          # a plan of 64-token tiles: the 64-token build takes its narrow-only list
+    (200, 3, 128, 256, 107, "200"),        # the same without wide tiles in the plan
 ])
 def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, seed, wide_bar):
     """A plan's 32-token tiles on a wide layer run on the 32-token build of the wide kernel (forced here
@@ -411,7 +413,7 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     qw, meta, s = make_deltas(N, k, m, seed)
     x = activations(T, k, seed + 1)
     idx = np.random.default_rng(seed + 2).integers(-1, N, size=T).astype(np.int32)
-    if wide_bar != "200":
+    if wide_bar != "200" and N >= 40:
         idx[: T // 3] = 1                                      # a hot delta: several wide tiles
     ref = orc.sbmm_4bit_2_4(qw, x, meta, s, idx)
     gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)

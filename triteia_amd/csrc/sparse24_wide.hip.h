@@ -25,8 +25,9 @@ namespace triteia_hip {
 constexpr int kWideTokens = 64;
 constexpr int kWideStages = 4;        // activation tiles in flight (LDS ring)
 
-// TOK: token rows of a tile (64, or 32 for the narrow tiles of a routing plan)
-template <int DEPTH, int TOK = kWideTokens>
+// TOK: token rows of a tile (64, or 32 for the narrow tiles of a routing plan).  PLAN_ALL: the kernel stands in
+// for the narrow kernel on a routing plan: it takes the plan's narrow tiles, or its narrow-only list.
+template <int DEPTH, int TOK = kWideTokens, bool PLAN_ALL = false>
 __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Args p) {
   constexpr int NT = TOK / 16;
   __shared__ __attribute__((aligned(1024))) _Float16 xs[kWideStages][TOK][128];
@@ -53,8 +54,8 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   bool alt_list = false;
   if (p.tiles) {
     int4 d = p.tiles[grp];
-    if (TOK == 32 && p.tiles_alt) {
-      // the 32-token build stands in for the narrow kernel on a plan's narrow tiles: like that kernel it takes
+    if (PLAN_ALL && p.tiles_alt) {
+      // this build stands in for the narrow kernel on a plan's narrow tiles: like that kernel it takes
       // the narrow-only list when the plan's wide tiles do not fill the chip (both candidates are requested together)
       const int4 d_alt = p.tiles_alt[grp];
       if ((long)p.n_groups_dev[4] * p.wide_gate < p.wide_min_units) {
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
     count = min(TOK, p.uniform_count - tc * TOK);
   }
   const int n_groups = p.n_groups_dev ? p.n_groups_dev[alt_list ? 5 : 0] : p.n_groups;
-  if (TOK != 32 && p.wide_min_units && (long)n_groups * p.wide_gate < p.wide_min_units) return;   // the narrow kernel has taken these tokens
+  if (!PLAN_ALL && p.wide_min_units && (long)n_groups * p.wide_gate < p.wide_min_units) return;   // the narrow kernel has taken these tokens
   if (grp >= n_groups) return;
   if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
   const int cnt = min(count, TOK);

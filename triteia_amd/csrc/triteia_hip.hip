@@ -350,9 +350,13 @@ constexpr int kPlanWideMinUnits = 200;
 // 24.9 -> 42.4 us).  The host only has the upper bound on the tiles; 600 on that bound separates the measured cases.
 constexpr int kMidMinUnits = 600;
 static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
-  if (!env_int("TRITEIA_HIP_MID", 1) || triteia_hip_plan_tile_tokens(prob_n, n_deltas) != 32) return false;
+  const int tile = triteia_hip_plan_tile_tokens(prob_n, n_deltas);
+  // (64-token plans as well, on the 64-token build, where K is short: cfg3 at 1024 / 2048 tokens 196 -> 170 /
+  // 250 -> 214 us; at k = 8192 the narrow kernel's workgroups live long enough: cfg4 at 2048 tokens 1478 -> 1523 us)
+  const bool mid64 = tile == 64 && env_int("TRITEIA_HIP_MID64", 1) && prob_k < env_int("TRITEIA_HIP_MID64_MAX_K", 8192);
+  if (!env_int("TRITEIA_HIP_MID", 1) || (tile != 32 && !mid64)) return false;
   if (prob_k % 128 != 0 || (long)prob_n * prob_k * 2 >= (1L << 32)) return false;   // whole K steps, 32-bit activation offsets
-  const long tiles = (n_deltas < prob_n ? n_deltas : prob_n) + prob_n / 32;
+  const long tiles = (n_deltas < prob_n ? n_deltas : prob_n) + prob_n / tile;
   return tiles * ((prob_m / 128 + 3) / 4) >= env_int("TRITEIA_HIP_MID_MIN_UNITS", kMidMinUnits);
 }
 constexpr int kFusedMaxTokens = 64 * kRawParts;   // kRawParts tokens per lane of a wavefront
@@ -434,9 +438,13 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
   if (mid) {
     const long cgs = (a.m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
     if ((long)a.n_groups * cg_pad > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units");
-    hipLaunchKernelGGL((sparse24_wide_kernel<1, 32>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), a);
-    if (int e = check_launch("sparse24_wide_kernel<32>")) return e;
+    if (tile == 32)
+      hipLaunchKernelGGL((sparse24_wide_kernel<1, 32, true>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
+                         static_cast<hipStream_t>(stream), a);
+    else
+      hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
+                         static_cast<hipStream_t>(stream), a);
+    if (int e = check_launch("sparse24_wide_kernel (plan tiles)")) return e;
   } else
   if (int e = launch_sparse24(a, pass_nt, tile / (16 * pass_nt), static_cast<hipStream_t>(stream))) return e;
   if (wide_launch) {
