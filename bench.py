@@ -324,6 +324,12 @@ def main():
             traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
         except Exception:
             traffic = None
+    # which kernel took the tiles (a plan's tiles on a wide layer run on a build of the wide kernel)
+    kernel_name = "sparse24_grouped_kernel"
+    if wl.indices is not None and not fused and not wl.index_offset:
+        tk = ffi.lib().triteia_hip_planned_tile_kernel(wl.tokens, wl.n_deltas, wl.m, wl.k)
+        if tk:
+            kernel_name = f"sparse24_wide_kernel<1, {tk}, true>"
     hbm_time, mfma_time = abytes / (HBM_PEAK_GBS * 1e9), wl.delta_flops() / (MFMA_SPARSE_F16_TFLOPS * 1e12)
     if mfma_time > hbm_time:
         # many tokens per delta: the matrix cores bound the kernel.  The 2:4-sparse instruction executes
@@ -340,7 +346,7 @@ def main():
     else:
         roofline = {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": traffic, "kernel": "sparse24_grouped_kernel", "kernel_us": round(kdur * 1e6, 2), "algorithmic_bytes": abytes,
+            "traffic": traffic, "kernel": kernel_name, "kernel_us": round(kdur * 1e6, 2), "algorithmic_bytes": abytes,
             "kernel_tflops": round(kflops, 2), "mfma_frac": round(kflops / MFMA_SPARSE_F16_TFLOPS, 4),
         }
 

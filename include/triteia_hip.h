@@ -131,6 +131,13 @@ TRITEIA_HIP_API int triteia_hip_route_plan(const void* token_indices, int index_
 
 TRITEIA_HIP_API int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas);
 
+/* Which kernel triteia_hip_sbmm_2_4_planned runs a plan's narrow tiles on for this batch and layer:
+ * 0 = the K-split narrow kernel (sparse24_grouped_kernel), 32 / 64 = the 32- / 64-token build of the
+ * wide kernel taking the plan's narrow-only list (wide layers; see the design notes).  No counterpart in
+ * the reference; for benchmarks and profiles, and for tests that compare results bit for bit (the two
+ * kernels add over K in different orders). */
+TRITEIA_HIP_API int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k);
+
 /* The multiply step alone, on a plan made by triteia_hip_route_plan for the same
  * (prob_n, n_deltas): C[t] (+)= A[t] @ dequant(B[d]) for every routed token.  One
  * plan serves every layer of a forward pass (the routing of a batch does not

@@ -365,6 +365,11 @@ static int plan_has_wide(int prob_n, int n_deltas) {
   return wide_enabled() && prob_n >= env_int("TRITEIA_HIP_WIDE_MIN_BATCH", 256) && prob_n >= 8 * groups;
 }
 
+int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
+  if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
+  return mid_tiles(prob_n, n_deltas, prob_m, prob_k) ? triteia_hip_plan_tile_tokens(prob_n, n_deltas) : 0;
+}
+
 int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
                            size_t workspace_bytes, int dev, void* stream) {
   if (prob_n < 0 || n_deltas < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "route_plan: tokens=%d deltas=%d", prob_n, n_deltas);
