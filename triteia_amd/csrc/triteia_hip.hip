@@ -357,6 +357,9 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (!env_int("TRITEIA_HIP_MID", 1) || (tile != 32 && !mid64)) return false;
   if (prob_k % 128 != 0 || (long)prob_n * prob_k * 2 >= (1L << 32)) return false;   // whole K steps, 32-bit activation offsets
   const long tiles = (n_deltas < prob_n ? n_deltas : prob_n) + prob_n / tile;
+  // (and only with a few tokens per tile at least: with two or three the shared activation tile saves nothing
+  // and the longer workgroups cost: 200 tokens over 65 of 512 resident deltas of 4096 x 11008 212 -> 238 us)
+  if (2 * prob_n < 7 * tiles) return false;
   return tiles * ((prob_m / 128 + 3) / 4) >= env_int("TRITEIA_HIP_MID_MIN_UNITS", kMidMinUnits);
 }
 constexpr int kFusedMaxTokens = 64 * kRawParts;   // kRawParts tokens per lane of a wavefront
