@@ -477,11 +477,14 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   // workgroups of the deltas without tokens make this form 1-2 % slower than a plan, which lists none)
   // (and from 128 tokens on, a batch whose deltas' weights are not requested ahead of the routing is better
   // off with a plan where the plan's tiles go to the 32-token wide kernel: 32 deltas of 4096 x 11008,
-  // 128 / 256 tokens: 69 -> 65.5 / 96 -> 89.5 us including the plan)
+  // 128 / 256 tokens: 69 -> 65.5 / 96 -> 89.5 us including the plan; on very large layers (k x m >= 2^27) a
+  // plan pays from 128 tokens on whatever the number of deltas, the plan launch being small against the kernel
+  // and the wide kernels taking hot deltas: 8 / 4 deltas of 8192 x 28672 with 128 / 256 tokens 145 -> 130 /
+  // 160 -> 122 us, while 8 or 16 deltas of 4096 x 11008 stay 8-12 % faster routed inside the kernel)
   const bool eager_ok = n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && env_int("TRITEIA_HIP_EAGER", 1);
   if (prob_n <= env_int("TRITEIA_HIP_FUSED_MAX_TOKENS", kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
       n_deltas <= (prob_n > 64 ? 32 : 64) && env_int("TRITEIA_HIP_FUSED_ROUTE", 1) &&
-      !(prob_n >= 128 && !eager_ok && mid_tiles(prob_n, n_deltas, prob_m, prob_k))) {
+      !(prob_n >= 128 && ((!eager_ok && mid_tiles(prob_n, n_deltas, prob_m, prob_k)) || (long)prob_k * prob_m >= (1L << 27)))) {
     // small batch: the multiply kernel routes by itself, no plan, no workspace traffic
     if (!token_indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null indices");
     DeviceGuard g(dev);
