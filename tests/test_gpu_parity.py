@@ -421,6 +421,7 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     for mid in ("1", "0"):
         monkeypatch.setenv("TRITEIA_HIP_MID", mid)
         monkeypatch.setenv("TRITEIA_HIP_MID_MIN_UNITS", "1")
+        monkeypatch.setenv("TRITEIA_HIP_MID_MIN_COLUMN_GROUPS", "1")
         out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
         sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
         torch.cuda.synchronize()

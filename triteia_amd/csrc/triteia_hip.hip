@@ -360,7 +360,11 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   // (and only with a few tokens per tile at least: with two or three the shared activation tile saves nothing
   // and the longer workgroups cost: 200 tokens over 65 of 512 resident deltas of 4096 x 11008 212 -> 238 us)
   if (2 * prob_n < 7 * tiles) return false;
-  return tiles * ((prob_m / 128 + 3) / 4) >= env_int("TRITEIA_HIP_MID_MIN_UNITS", kMidMinUnits);
+  // (and a layer of 16 column groups at least: on m = 4096 it is even at best, 64 deltas with 8 tokens each 80 us
+  // both ways, and loses with few tokens per tile, 128 deltas with 6 each 146 -> 164 us)
+  const long cgs = (prob_m / 128 + 3) / 4;
+  if (cgs < env_int("TRITEIA_HIP_MID_MIN_COLUMN_GROUPS", 16)) return false;
+  return tiles * cgs >= env_int("TRITEIA_HIP_MID_MIN_UNITS", kMidMinUnits);
 }
 constexpr int kFusedMaxTokens = 64 * kRawParts;   // kRawParts tokens per lane of a wavefront
 static int plan_has_wide(int prob_n, int n_deltas) {
