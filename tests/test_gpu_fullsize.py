@@ -162,6 +162,31 @@ def test_bmm_many_tokens_per_matrix(ops):
         assert float(err) <= 2e-3
 
 
+def test_activations_above_4_gib(ops):
+    """The wide kernels address activations with 32-bit byte offsets; a batch whose activations reach
+    4 GiB must be kept away from them (and from every other 32-bit shortcut) by the launcher."""
+    from triteia_amd.python.capi import routed_workspace, sbmm_2_4_routed
+    from triteia_amd.python.ops.utils.sparsity import unpack_2_4
+    T, k, m, N = 2 ** 18 + 64, 8192, 128, 2
+    say(f"activations of {T * k * 2 / 2 ** 30:.3f} GiB: matmul, then routed over {N} deltas")
+    q, me, s = W.random_packed_deltas(N, k, m, 91, DEV)
+    x = torch.randn((T, k), generator=torch.Generator(device=DEV).manual_seed(92), device=DEV, dtype=torch.float16)
+    dense = [unpack_2_4(q[i], me[i], s[i]).float() for i in range(N)]
+    out = ops.matmul_4bit_2_4(q[0], x, me[0], s[0])
+    idx = np.random.default_rng(93).integers(-1, N, size=T).astype(np.int32)
+    gi = torch.from_numpy(idx).to(DEV)
+    got = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
+    sbmm_2_4_routed(x, q, me, got, s, gi, accumulate=False, workspace=routed_workspace(T, N, DEV))
+    assert bool((got[gi < 0] == -3.0).all())
+    for a in range(0, T, 32768):          # fp32 references in chunks of the batch
+        xx = x[a:a + 32768].float()
+        r0, r1 = xx @ dense[0], xx @ dense[1]
+        assert float((out[a:a + 32768].float() - r0).norm() / r0.norm()) <= 2e-3, f"matmul rows {a}.."
+        g = gi[a:a + 32768]
+        ref, sel = torch.where((g == 0)[:, None], r0, r1), g >= 0
+        assert float((got[a:a + 32768][sel].float() - ref[sel]).norm() / ref[sel].norm()) <= 2e-3, f"routed rows {a}.."
+
+
 def test_reference_import_path_alias():
     import triteia.python.ops as ref_ops
     from triteia.python.capi import mul_2_4  # noqa: F401
