@@ -107,3 +107,37 @@ def test_ldmm_replays():
         assert torch.equal(replayed, result), f"replay {rep} differs from the eager call"
         y0 = torch.matmul(x, gb.t()).float().cpu().numpy().astype(np.float64)
         check_close(replayed, y0 + orc.ldmm(hidx, hx, A, B, qw, meta, s), what=f"ldmm replay {rep}")
+
+
+def test_matmul_and_bmm_replay():
+    """The uniform entry points (one to three launches each: wide tiles, a narrow rest) in one graph."""
+    from triteia_amd.python import ops
+    T, B, t, k, m, seed = 300, 3, 40, 512, 1024, 221
+    print(f"[case] graph replay of matmul T={T} and bmm {B} x {t}, k={k} m={m}", flush=True)
+    qw, meta, s = make_deltas(B, k, m, seed)
+    gq, gm, gs = to_gpu(qw, meta, s)
+    x = torch.zeros((T, k), dtype=torch.float16, device=DEV)
+    xb = torch.zeros((B, t, k), dtype=torch.float16, device=DEV)
+    y = torch.zeros((T, m), dtype=torch.float16, device=DEV)
+    yb = torch.zeros((B, t, m), dtype=torch.float16, device=DEV)
+
+    def step():
+        y.copy_(ops.matmul_4bit_2_4(gq[0], x, gm[0], gs[0]))
+        yb.copy_(ops.bmm_4bit_2_4(gq, xb, gm, gs))
+
+    step()
+    torch.cuda.synchronize()
+    graph = _capture(step)
+    for rep in range(3):
+        hx, hxb = activations(T, k, seed + 10 + rep), activations(B * t, k, seed + 20 + rep).reshape(B, t, k)
+        x.copy_(torch.from_numpy(hx))
+        xb.copy_(torch.from_numpy(hxb))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ry, ryb = y.clone(), yb.clone()
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(ry, y) and torch.equal(ryb, yb), f"replay {rep} differs from the eager call"
+        check_close(ry, orc.matmul_4bit_2_4(qw[0], hx, meta[0], s[0]), what=f"matmul replay {rep}")
+        check_close(ryb, orc.bmm_4bit_2_4(qw, hxb, meta, s), what=f"bmm replay {rep}")
