@@ -61,7 +61,7 @@ def test_matmul_4bit_2_4(ops, n, k, m, seed):
     check_close(out, ref, what="matmul_4bit_2_4")
 
 
-@pytest.mark.parametrize("kernel", ["wide64", "wide128"])
+@pytest.mark.parametrize("kernel", ["wide64", "wide128", "wide32"])
 @pytest.mark.parametrize("n,k,m,seed", [
     (64, 128, 512, 21), (128, 128, 512, 22), (128, 256, 128, 23),      # one tile, 1 and 2 k steps
     (200, 384, 384, 24), (321, 512, 640, 25), (130, 640, 256, 26),     # ragged tokens, partial column groups
@@ -69,13 +69,16 @@ def test_matmul_4bit_2_4(ops, n, k, m, seed):
     (192, 192, 256, 29),                                               # k = 64 (mod 128): falls back to the narrow kernel
 ])
 def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
-    """The matrix-core-bound kernels (64- and 128-token tiles), forced onto small ragged
-    shapes that the launcher would give to the narrow kernel."""
+    """The matrix-core-bound kernels (64- and 128-token tiles) and the 32-token build with two steps of
+    weights in flight, forced onto small ragged shapes that the launcher would give to the narrow kernel."""
     say(f"matmul {kernel} n={n} k={k} m={m} seed={seed}")
     monkeypatch.setenv("TRITEIA_HIP_WIDE_MIN_UNITS", "1")
     monkeypatch.setenv("TRITEIA_HIP_WIDE128_MIN_UNITS", "1")
     monkeypatch.setenv("TRITEIA_HIP_WIDE128_MIN_K", "0")
     monkeypatch.setenv("TRITEIA_HIP_WIDE128", "1" if kernel == "wide128" else "0")
+    if kernel == "wide32":      # takes the tokens ahead of the other two whenever its window of units is open
+        monkeypatch.setenv("TRITEIA_HIP_WIDE32_MIN_UNITS", "1")
+        monkeypatch.setenv("TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")
     qw, meta, s = make_deltas(1, k, m, seed)
     x = activations(n, k, seed + 1)
     ref = orc.matmul_4bit_2_4(qw[0], x, meta[0], s[0])
@@ -165,6 +168,28 @@ def test_bmm_4bit_2_4(ops, b, t, k, m, seed):
     # does, so the two differ in the order of fp32 accumulation only
     assert float((out.float() - loop.float()).norm() / loop.float().norm()) < 1e-4
     assert orc.rel_mean_abs(out.float().cpu().numpy(), ref) < max(tol, 1e-3)
+
+
+@pytest.mark.parametrize("b,t,k,m,seed", [
+    (3, 70, 384, 640, 31),     # two full tiles per matrix and a last one of 6 tokens
+    (2, 50, 256, 1152, 32),    # a last tile of 18 tokens
+    (5, 32, 128, 128, 33),     # one tile, one step, one column block
+])
+def test_bmm_32_token_wide_kernel(ops, monkeypatch, b, t, k, m, seed):
+    """Uniform groups on the 32-token build of the wide kernel (by default only for launches of 176 to 512 units)."""
+    say(f"bmm on 32-token wide tiles b={b} t={t} k={k} m={m} seed={seed}")
+    monkeypatch.setenv("TRITEIA_HIP_WIDE32_MIN_UNITS", "1")
+    monkeypatch.setenv("TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")
+    qw, meta, s = make_deltas(b, k, m, seed)
+    x = activations(b * t, k, seed + 1).reshape(b, t, k)
+    gq, gm, gs, gx = to_gpu(qw, meta, s, x)
+    out = ops.bmm_4bit_2_4(gq, gx, gm, gs)
+    torch.cuda.synchronize()
+    check_close(out, orc.bmm_4bit_2_4(qw, x, meta, s), what="bmm on 32-token wide tiles")
+    monkeypatch.setenv("TRITEIA_HIP_WIDE", "0")
+    narrow = ops.bmm_4bit_2_4(gq, gx, gm, gs)
+    torch.cuda.synchronize()
+    assert float((out.float() - narrow.float()).norm() / narrow.float().norm()) < 1e-4
 
 
 # -------------------------------------------------------------------- sbmm

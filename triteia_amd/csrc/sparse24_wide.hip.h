@@ -25,8 +25,9 @@ namespace triteia_hip {
 constexpr int kWideTokens = 64;
 constexpr int kWideStages = 4;        // activation tiles in flight (LDS ring)
 
-// TOK: token rows of a tile (64, or 32 for the narrow tiles of a routing plan).  PLAN_ALL: the kernel stands in
-// for the narrow kernel on a routing plan: it takes the plan's narrow tiles, or its narrow-only list.
+// TOK: token rows of a tile (64, or 32 for the narrow tiles of a routing plan and for uniform groups in launches
+// that do not fill the chip).  PLAN_ALL: the kernel stands in for the narrow kernel on a routing plan: it takes the
+// plan's narrow tiles, or its narrow-only list.  DEPTH: steps of weights in flight per wavefront.
 template <int DEPTH, int TOK = kWideTokens, bool PLAN_ALL = false>
 __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Args p) {
   constexpr int NT = TOK / 16;

@@ -169,17 +169,20 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
 }
 
 
-// Wide (64-token x 512-column) tiles: groups from a plan's wide list or uniform groups.
-int launch_wide(const Sparse24Args& a, hipStream_t st) {
+// Wide (64-token x 512-column) tiles: groups from a plan's wide list or uniform groups.  `tok` = 32: uniform groups
+// in 32-token tiles on the 32-token build with two steps of weights in flight (launches that do not fill the chip).
+int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   const long cgs = (a.m / 128 + 3) / 4;
   const long cg_pad = (cgs + 7) / 8 * 8;
-  const long chunks = a.tiles ? 1 : (a.uniform_count + kWideTokens - 1) / kWideTokens;
+  const long chunks = a.tiles ? 1 : (a.uniform_count + tok - 1) / tok;
   const long units = (long)a.n_groups * chunks * cg_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   Sparse24Args b = a;
   if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
-  if (env_int("TRITEIA_HIP_WIDE_DEPTH", 1) == 1)
+  if (tok == 32)
+    hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false>), dim3((unsigned)units), dim3(256), 0, st, b);
+  else if (env_int("TRITEIA_HIP_WIDE_DEPTH", 1) == 1)
     hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3((unsigned)units), dim3(256), 0, st, b);
   else
     hipLaunchKernelGGL((sparse24_wide_kernel<2>), dim3((unsigned)units), dim3(256), 0, st, b);
@@ -214,6 +217,7 @@ bool wide_enabled() { return env_int("TRITEIA_HIP_WIDE", 1) != 0; }
 bool wide128_enabled() { return wide_enabled() && env_int("TRITEIA_HIP_WIDE128", 0) != 0; }
 constexpr long kWideMinUnits = 160;   // 4096 x 4096: 1024 tokens (128 tiles) 54.9 us wide against 46.5 us narrow, 1536 tokens (192) 60.8 against 71.1
 constexpr long kWide128MinUnits = 192;
+constexpr long kWide32MinUnits = 176, kWide32MaxUnits = 448;   // (32-token tile, 512-column group) units: see launch_uniform
 
 // `tokens` rows per group, `stride` rows between groups: the head of each group goes to the
 // 128-token kernel, then to the 64-token kernel (full tiles, and a rest above half a tile),
@@ -226,9 +230,30 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   int done = 0;
   // (the wide kernels address activations with 32-bit byte offsets)
   const bool x_below_4g = ((long)(n_groups - 1) * stride + tokens) * a.x_stride * 2 < (1L << 32);
+  // A launch of at most two 32-token workgroups per CU, but of more than the narrow kernel fills well, is bound by
+  // the latency of each workgroup's chain of steps, not by the matrix cores: there the 32-token build of the wide
+  // kernel with two steps of weights in flight per wavefront beats both the narrow kernel and 64-token tiles.
+  // Measured (narrow or 64-token -> this): 4096 x 4096 with 640 / 1024 / 1536 / 2048 tokens 45.7 -> 37.2, 46.5 -> 38.2,
+  // 54.5 -> 49.7, 60.8 -> 55.6 us; 4096 x 11008 with 384 / 512 tokens 66 -> 46.7, 54.7 -> 48.5 us; 8192 x 8192 with
+  // 384 / 768 tokens 76.5 -> 66.5, 94.7 -> 86.9 us; 8192 x 28672 with 128 / 256 tokens 79 -> 69.3, 99.5 -> 95.5 us.
+  // Outside the window it loses: 8192 x 28672 with 96 tokens (168 units) 64 -> 69 us, 4096 x 11008 with 768 tokens
+  // (528 units) 64 -> 76 us.
+  {
+    // (a last tile of any size counts: in a launch of one round its workgroups cost nothing, a separate launch of
+    // the narrow kernel for them streams the weights once more)
+    const long units32 = (long)n_groups * ((tokens + 31) / 32) * cgs;
+    if (wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= 32 &&
+        units32 >= env_int("TRITEIA_HIP_WIDE32_MIN_UNITS", kWide32MinUnits) &&
+        units32 <= env_int("TRITEIA_HIP_WIDE32_MAX_UNITS", kWide32MaxUnits)) {
+      a.uniform_first = 0;
+      a.uniform_count = tokens;
+      if (int e = launch_wide(a, st, 32)) return e;
+      done = tokens;
+    }
+  }
   // (the 128-token kernel pays from k = 8192 on: 2-3 % faster than the 64-token kernel at 8192 x 8192 and
   // 8192 x 28672, 4-8 % slower at 4096 x 4096 and 4096 x 11008, whose K loops are too short for its pipeline)
-  if (wide128_enabled() && a.k % 128 == 0 && a.k >= env_int("TRITEIA_HIP_WIDE128_MIN_K", 8192) && x_below_4g &&
+  if (done == 0 && wide128_enabled() && a.k % 128 == 0 && a.k >= env_int("TRITEIA_HIP_WIDE128_MIN_K", 8192) && x_below_4g &&
       (long)n_groups * (tokens / kWide128Tokens) * cgs >= env_int("TRITEIA_HIP_WIDE128_MIN_UNITS", kWide128MinUnits)) {
     int t = tokens / kWide128Tokens * kWide128Tokens;
     if (tokens - t > kWideTokens) t = tokens;
@@ -242,7 +267,12 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
       (done > 0 ? rest >= kPlanWideMinRest
                 : (long)n_groups * (rest / kWideTokens) * cgs >= env_int("TRITEIA_HIP_WIDE_MIN_UNITS", kWideMinUnits))) {
     int t = rest / kWideTokens * kWideTokens;
-    if (rest - t >= kPlanWideMinRest) t = rest;
+    // A rest above half a tile becomes a tile of its own; a smaller one too while the launch stays within one
+    // round of workgroups (two per CU), where its workgroups cost nothing and a launch of the narrow kernel for them
+    // would stream the weights once more (288 tokens on 8192 x 28672: 130.6 -> 111.5 us; 2056 on 4096 x 4096 69.3 ->
+    // 67.4 us).  Past one round the extra tile starts a round of its own (4104 tokens on 4096 x 4096: 88 -> 111 us).
+    const bool one_round = (long)n_groups * (rest / kWideTokens + 1) * cgs <= 512;
+    if (rest - t >= (one_round ? 1 : kPlanWideMinRest)) t = rest;
     a.uniform_first = done;
     a.uniform_count = t;
     if (int e = launch_wide(a, st)) return e;
