@@ -121,7 +121,7 @@ TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n
  *   int32 all[max_tiles][4]   = at the next multiple of 4 ints: for plans with wide tiles, the
  *         same tokens cut into narrow tiles only (header[5] of them).  The multiply kernels pick
  *         {tiles, wide} or {all} per weight shape on the device: the wide kernel runs only if
- *         its tiles fill the chip (wide tiles x ceil(prob_m / 512) >= 200, environment
+ *         its tiles fill the chip (wide tiles x ceil(prob_m / 512) >= 150, environment
  *         TRITEIA_HIP_PLAN_WIDE_MIN_UNITS); the LoRA path always takes all[].
  * with max_tiles = min(prob_n, n_deltas) + prob_n / 16 and max_wide = prob_n / 33 + 1.  The
  * narrow tile size is triteia_hip_plan_tile_tokens(prob_n, n_deltas).  Exposed so that one

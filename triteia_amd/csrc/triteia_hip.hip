@@ -371,7 +371,9 @@ int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas) {
 // the wide kernel takes its tiles only if they fill the chip (wide tiles x column groups of the
 // layer >= kPlanWideMinUnits); otherwise re-reading a hot delta's weights from cache in narrow
 // tiles is cheaper than a second, poorly filled launch, and the wide launch returns at once.
-constexpr int kPlanWideMinUnits = 200;
+// (measured between the two: launches of 152-176 wide units are 16-23 % faster on the wide kernel, 4 deltas of 4096 x 11008
+// with 512 tokens 73 -> 61 us, 2 of 8192 x 8192 with 640 tokens 118 -> 99 us; launches of 128 are 12-20 % slower there)
+constexpr int kPlanWideMinUnits = 150;
 // A plan's 32-token tiles on a wide layer go to the 32-token build of the wide kernel (four column blocks of a
 // workgroup share each activation tile through LDS, every wavefront walks all of K) instead of the K-split narrow
 // kernel, whose column-block workgroups each fetch the tile's activations again: 5-10 % faster once there are
