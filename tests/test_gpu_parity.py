@@ -176,7 +176,7 @@ def test_bmm_4bit_2_4(ops, b, t, k, m, seed):
     (5, 32, 128, 128, 33),     # one tile, one step, one column block
 ])
 def test_bmm_32_token_wide_kernel(ops, monkeypatch, b, t, k, m, seed):
-    """Uniform groups on the 32-token build of the wide kernel (by default only for launches of 176 to 512 units)."""
+    """Uniform groups on the 32-token build of the wide kernel (by default only for launches of 160 to 448 units)."""
     say(f"bmm on 32-token wide tiles b={b} t={t} k={k} m={m} seed={seed}")
     monkeypatch.setenv("TRITEIA_HIP_WIDE32_MIN_UNITS", "1")
     monkeypatch.setenv("TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")

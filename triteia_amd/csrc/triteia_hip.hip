@@ -217,7 +217,7 @@ bool wide_enabled() { return env_int("TRITEIA_HIP_WIDE", 1) != 0; }
 bool wide128_enabled() { return wide_enabled() && env_int("TRITEIA_HIP_WIDE128", 0) != 0; }
 constexpr long kWideMinUnits = 160;   // 4096 x 4096: 1024 tokens (128 tiles) 54.9 us wide against 46.5 us narrow, 1536 tokens (192) 60.8 against 71.1
 constexpr long kWide128MinUnits = 192;
-constexpr long kWide32MinUnits = 176, kWide32MaxUnits = 448;   // (32-token tile, 512-column group) units: see launch_uniform
+constexpr long kWide32MinUnits = 160, kWide32MaxUnits = 448;   // (32-token tile, 512-column group) units: see launch_uniform
 
 // `tokens` rows per group, `stride` rows between groups: the head of each group goes to the
 // 128-token kernel, then to the 64-token kernel (full tiles, and a rest above half a tile),
@@ -236,8 +236,10 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   // Measured (narrow or 64-token -> this): 4096 x 4096 with 640 / 1024 / 1536 / 2048 tokens 45.7 -> 37.2, 46.5 -> 38.2,
   // 54.5 -> 49.7, 60.8 -> 55.6 us; 4096 x 11008 with 384 / 512 tokens 66 -> 46.7, 54.7 -> 48.5 us; 8192 x 8192 with
   // 384 / 768 tokens 76.5 -> 66.5, 94.7 -> 86.9 us; 8192 x 28672 with 128 / 256 tokens 79 -> 69.3, 99.5 -> 95.5 us.
-  // Outside the window it loses: 8192 x 28672 with 96 tokens (168 units) 64 -> 69 us, 4096 x 11008 with 768 tokens
-  // (528 units) 64 -> 76 us.
+  // At 160 units: 4096 x 4096 with 640 tokens 45 -> 36.7, 8192 x 8192 with 320 tokens 76.5 -> 66.2, 11008 x 4096 with 640
+  // tokens 98.8 -> 89.5 us.  Outside the window it loses: 8192 x 8192 with 288 tokens (144 units) 61.7 -> 65.7 us,
+  // 4096 x 11008 with 160 tokens (110 units) 28.9 -> 37 us, with 768 tokens (528 units) 64 -> 76 us; inside it one
+  // case measured slower: 8192 x 28672 with 96 tokens (168 units) 64 -> 69 us.
   {
     // (a last tile of any size counts: in a launch of one round its workgroups cost nothing, a separate launch of
     // the narrow kernel for them streams the weights once more)
