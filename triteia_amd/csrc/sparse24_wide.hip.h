@@ -28,14 +28,18 @@ constexpr int kWideStages = 4;        // activation tiles in flight (LDS ring)
 // TOK: token rows of a tile (64, or 32 for the narrow tiles of a routing plan and for uniform groups in launches
 // that do not fill the chip).  PLAN_ALL: the kernel stands in for the narrow kernel on a routing plan: it takes the
 // plan's narrow tiles, or its narrow-only list.  DEPTH: steps of weights in flight per wavefront.
-template <int DEPTH, int TOK = kWideTokens, bool PLAN_ALL = false>
-__global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Args p) {
+// KS = 2: eight wavefronts; wavefronts 4..7 take the second half of the K steps of the same four column blocks (an
+// activation ring of their own) and hand their sums to wavefronts 0..3 through LDS at the end: half as long a chain
+// of steps per wavefront, for launches of at most one workgroup per CU.
+template <int DEPTH, int TOK = kWideTokens, bool PLAN_ALL = false, int KS = 1>
+__global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kernel(const Sparse24Args p) {
   constexpr int NT = TOK / 16;
-  __shared__ __attribute__((aligned(1024))) _Float16 xs[kWideStages][TOK][128];
+  __shared__ __attribute__((aligned(1024))) _Float16 xs[KS][kWideStages][TOK][128];
   __shared__ int s_rows[TOK];
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
+  const int wave = (tid >> 6) & 3;   // column block of the group
+  const int kh = KS == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);   // half of K (KS = 2); wave-uniform
   const int lane = tid & 63;
   const int r = lane & 15;
   const int q = lane >> 4;
@@ -85,7 +89,11 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   const int cbc = active ? cb : col_blocks - 1;  // idle waves still run the barriers
 
   const int k_rows = p.k >> 5;
-  const int n_steps = (k_rows + 3) >> 2;
+  const int all_steps = (k_rows + 3) >> 2;
+  // this wavefront's steps: [step0, step0 + n_steps); every wavefront runs `loop_steps` rounds of the loop (barriers)
+  const int loop_steps = (all_steps + KS - 1) / KS;
+  const int step0 = kh == 0 ? 0 : loop_steps;
+  const int n_steps = kh == 0 ? loop_steps : all_steps - loop_steps;
   const long qrow = p.m >> 1;
   const long mrow = p.m >> 2;
   // operand addresses = a base that is the same for the whole wave (scalar registers) + a 32-bit byte
@@ -118,9 +126,9 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   // the first LDS read behind it must complete, i.e. it drains every outstanding request (the
   // weights requested a moment ago included) once per K step.  The LDS address of a request is
   // M0 + 16 * lane.
-  const uint32_t lds_x_wave = (uint32_t)(uintptr_t)&xs[0][4 * wave][0];
+  const uint32_t lds_x_wave = (uint32_t)(uintptr_t)&xs[kh][0][4 * wave][0];
   auto issue_x = [&](int st) {
-    const int stc = min(st, n_steps - 1);   // past the end: refetch the last tile (never read)
+    const int stc = min(step0 + min(st, n_steps - 1), all_steps - 1);   // past the end: refetch a valid tile (never read)
     const int stage = st & (kWideStages - 1);
 #pragma unroll
     for (int ii = 0; ii < NT; ii++) {
@@ -135,7 +143,7 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
     uint4_t mt[2];
   };
   auto load_w = [&](WFrag& f, int st) {
-    const long tr0 = (st < n_steps ? st : 0) << 2;   // past the end: any valid rows (never used); k % 128 == 0, so
+    const long tr0 = (st < n_steps ? step0 + st : 0) << 2;   // past the end: any valid rows (never used); k % 128 == 0, so
     const char* wb = reinterpret_cast<const char*>(qw_delta + tr0 * qrow);   // rows tr0 .. tr0 + 3 always exist
     const char* mb = reinterpret_cast<const char*>(mt_delta + tr0 * mrow);
 #pragma unroll
@@ -157,7 +165,7 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   auto read_b = [&](int stage, int nt, int u) {
     // chunks c and c + 8 of token row nt*16 + r, at their swizzled positions
     const int c = (xb_off >> 3) + 2 * u;
-    const _Float16* row = &xs[stage][nt * 16 + r][0];
+    const _Float16* row = &xs[kh][stage][nt * 16 + r][0];
     typedef uint32_t uint8_t_v __attribute__((ext_vector_type(8)));
     const uint4_t lo = *reinterpret_cast<const uint4_t*>(row + ((c ^ r) << 3));
     const uint4_t hi = *reinterpret_cast<const uint4_t*>(row + (((c + 8) ^ r) << 3));
@@ -227,7 +235,7 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
 #pragma unroll
   for (int j = 0; j < DEPTH; j++) load_w(ring[j], j);
   constexpr int TURN = DEPTH > 4 ? DEPTH : 4;   // whole ring turns of both rings (DEPTH divides 4)
-  for (int s0 = 0; s0 < n_steps; s0 += TURN) {
+  for (int s0 = 0; s0 < loop_steps; s0 += TURN) {
 #pragma unroll
     for (int j = 0; j < TURN; j++) {
       const int st = s0 + j;
@@ -240,6 +248,28 @@ __global__ __launch_bounds__(256, 2) void sparse24_wide_kernel(const Sparse24Arg
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive the block's LDS
 
+  if (KS == 2) {
+    // the second half's sums go to the first half through the memory of the activation rings (same size:
+    // 2048 * TOK bytes), register by register with consecutive lanes side by side
+    __syncthreads();   // every wavefront has read its last tile
+    float* red = reinterpret_cast<float*>(&xs[0][0][0][0]) + wave * (32 * NT * 64) + lane;
+    if (kh == 1) {
+#pragma unroll
+      for (int cc = 0; cc < 8; cc++)
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) red[((cc * NT + nt) * 4 + j) * 64] = acc[cc][nt][j];
+    }
+    __syncthreads();
+    if (kh == 1) return;
+#pragma unroll
+    for (int cc = 0; cc < 8; cc++)
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[cc][nt][j] += red[((cc * NT + nt) * 4 + j) * 64];
+  }
   if (!active) return;
   // epilogue: lane (n = r, qq = q) holds features 32q + 8j + c of token n for every 16-token tile
   const _Float16* sc = p.scales + (long)delta * p.scales_stride + cb * 128 + 32 * q;

@@ -169,6 +169,9 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
 }
 
 
+// 32-token launches of at most one workgroup per CU run with eight wavefronts per workgroup (K split in two inside the
+// workgroup): 20-27 % faster from 160 to 256 units, slower beyond (two rounds of workgroups that fill a CU each).
+constexpr long kWide32KSplitMaxUnits = 256;
 // Wide (64-token x 512-column) tiles: groups from a plan's wide list or uniform groups.  `tok` = 32: uniform groups
 // in 32-token tiles on the 32-token build with two steps of weights in flight (launches that do not fill the chip).
 int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
@@ -180,7 +183,9 @@ int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   Sparse24Args b = a;
   if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
-  if (tok == 32)
+  if (tok == 32 && units <= env_int("TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS", kWide32KSplitMaxUnits))
+    hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false, 2>), dim3((unsigned)units), dim3(512), 0, st, b);
+  else if (tok == 32)
     hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false>), dim3((unsigned)units), dim3(256), 0, st, b);
   else if (env_int("TRITEIA_HIP_WIDE_DEPTH", 1) == 1)
     hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3((unsigned)units), dim3(256), 0, st, b);
