@@ -61,7 +61,7 @@ def test_matmul_4bit_2_4(ops, n, k, m, seed):
     check_close(out, ref, what="matmul_4bit_2_4")
 
 
-@pytest.mark.parametrize("kernel", ["wide64", "wide128", "wide32", "wide32ks"])
+@pytest.mark.parametrize("kernel", ["wide64", "wide64ks", "wide128", "wide32", "wide32ks"])
 @pytest.mark.parametrize("n,k,m,seed", [
     (64, 128, 512, 21), (128, 128, 512, 22), (128, 256, 128, 23),      # one tile, 1 and 2 k steps
     (200, 384, 384, 24), (321, 512, 640, 25), (130, 640, 256, 26),     # ragged tokens, partial column groups
@@ -81,6 +81,7 @@ def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
         monkeypatch.setenv("TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")
     # wide32ks: eight wavefronts per workgroup, each half of them on half of the k steps
     monkeypatch.setenv("TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS", "1000000000" if kernel == "wide32ks" else "0")
+    monkeypatch.setenv("TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS", "1000000000" if kernel == "wide64ks" else "0")
     qw, meta, s = make_deltas(1, k, m, seed)
     x = activations(n, k, seed + 1)
     ref = orc.matmul_4bit_2_4(qw[0], x, meta[0], s[0])

@@ -172,6 +172,9 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
 // 32-token launches of at most one workgroup per CU run with eight wavefronts per workgroup (K split in two inside the
 // workgroup): 20-27 % faster from 160 to 256 units, slower beyond (two rounds of workgroups that fill a CU each).
 constexpr long kWide32KSplitMaxUnits = 256;
+// The same for 64-token tiles (256 registers, 128 KiB of LDS): 9-20 % faster than the 32-token build with four wavefronts
+// at 257-448 of its units and than the 64-token build with four wavefronts up to 256 units (one workgroup per CU).
+constexpr long kWide64KSplitMaxUnits = 256;
 // Wide (64-token x 512-column) tiles: groups from a plan's wide list or uniform groups.  `tok` = 32: uniform groups
 // in 32-token tiles on the 32-token build with two steps of weights in flight (launches that do not fill the chip).
 int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
@@ -187,6 +190,9 @@ int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
     hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false, 2>), dim3((unsigned)units), dim3(512), 0, st, b);
   else if (tok == 32)
     hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false>), dim3((unsigned)units), dim3(256), 0, st, b);
+  else if (units <= env_int("TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS", kWide64KSplitMaxUnits) &&
+           !a.tiles)   // (a plan's launch is sized by an upper bound on its tiles; at 190-230 real units it measured the same either way)
+    hipLaunchKernelGGL((sparse24_wide_kernel<1, kWideTokens, false, 2>), dim3((unsigned)units), dim3(512), 0, st, b);
   else if (env_int("TRITEIA_HIP_WIDE_DEPTH", 1) == 1)
     hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3((unsigned)units), dim3(256), 0, st, b);
   else
@@ -233,6 +239,7 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   a.delta_step = delta_step;
   const long cgs = (a.m / 128 + 3) / 4;
   int done = 0;
+  bool ks64 = false;   // the whole launch goes to 64-token tiles on workgroups of eight wavefronts
   // (the wide kernels address activations with 32-bit byte offsets)
   const bool x_below_4g = ((long)(n_groups - 1) * stride + tokens) * a.x_stride * 2 < (1L << 32);
   // A launch of at most two 32-token workgroups per CU, but of more than the narrow kernel fills well, is bound by
@@ -249,7 +256,15 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
     // (a last tile of any size counts: in a launch of one round its workgroups cost nothing, a separate launch of
     // the narrow kernel for them streams the weights once more)
     const long units32 = (long)n_groups * ((tokens + 31) / 32) * cgs;
-    if (wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= 32 &&
+    // past the launches that the 32-token build runs with eight wavefronts, 64-token tiles with eight wavefronts
+    // are ahead while they make one workgroup per CU at most (4096 x 4096 with 1280 / 1536 tokens 49.7 -> 44.2,
+    // 50.8 -> 46.0 us; 4096 x 11008 with 384 / 640 tokens 47.2 -> 43.0, 51.4 -> 46.0 us; 8192 x 8192 with 768 tokens 88.7 ->
+    // 72.5 us; 8192 x 28672 with 192 tokens 89.4 -> 73.0 us)
+    ks64 = wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= kWideTokens &&
+           units32 > env_int("TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS", kWide32KSplitMaxUnits) &&
+           (long)n_groups * ((tokens + kWideTokens - 1) / kWideTokens) * ((cgs + 7) / 8 * 8) <=
+               env_int("TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS", kWide64KSplitMaxUnits);
+    if (!ks64 && wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= 32 &&
         units32 >= env_int("TRITEIA_HIP_WIDE32_MIN_UNITS", kWide32MinUnits) &&
         units32 <= env_int("TRITEIA_HIP_WIDE32_MAX_UNITS", kWide32MaxUnits)) {
       a.uniform_first = 0;
@@ -272,7 +287,7 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   int rest = tokens - done;
   if (rest > 0 && wide_enabled() && a.k % 128 == 0 && x_below_4g &&
       (done > 0 ? rest >= kPlanWideMinRest
-                : (long)n_groups * (rest / kWideTokens) * cgs >= env_int("TRITEIA_HIP_WIDE_MIN_UNITS", kWideMinUnits))) {
+                : ks64 || (long)n_groups * (rest / kWideTokens) * cgs >= env_int("TRITEIA_HIP_WIDE_MIN_UNITS", kWideMinUnits))) {
     int t = rest / kWideTokens * kWideTokens;
     // A rest above half a tile becomes a tile of its own; a smaller one too while the launch stays within one
     // round of workgroups (two per CU), where its workgroups cost nothing and a launch of the narrow kernel for them
