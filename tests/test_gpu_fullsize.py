@@ -162,6 +162,30 @@ def test_bmm_many_tokens_per_matrix(ops):
         assert float(err) <= 2e-3
 
 
+@pytest.mark.parametrize("b,t,k,m", [
+    (1, 1024, 4096, 4096),    # 256 units of 32 tokens: 32-token tiles, K split over eight wavefronts
+    (1, 1500, 4096, 4096),    # 192 units of 64 tokens, last tile of 28: 64-token tiles, K split over eight wavefronts
+    (2, 200, 4096, 11008),    # two matrices, 4 tiles each with a last one of 8 tokens, 22 column groups padded to 24
+    (1, 576, 8192, 8192),     # 144 units of 64 tokens, 64 steps per half
+])
+def test_uniform_launches_of_one_workgroup_per_cu(ops, monkeypatch, b, t, k, m):
+    """The launcher's own choice for launches that do not fill the chip (workgroups of eight wavefronts, each half
+    on half of the K steps) against a dequantise-then-matmul in fp32 and against the narrow kernel."""
+    say(f"bmm {b} x {t} tokens, {k} x {m}: default launch rule")
+    from triteia_amd.python.ops.utils.sparsity import unpack_2_4
+    q, me, s = W.random_packed_deltas(b, k, m, 91, DEV)
+    x = W.random_activations(b * t, k, 92, DEV).reshape(b, t, k)
+    out = ops.bmm_4bit_2_4(q, x, me, s)
+    torch.cuda.synchronize()
+    for i in range(b):
+        ref = x[i].float() @ unpack_2_4(q[i], me[i], s[i]).float()
+        assert float((out[i].float() - ref).norm() / ref.norm()) <= 2e-3
+    monkeypatch.setenv("TRITEIA_HIP_WIDE", "0")
+    narrow = ops.bmm_4bit_2_4(q, x, me, s)
+    torch.cuda.synchronize()
+    assert float((out.float() - narrow.float()).norm() / narrow.float().norm()) < 1e-4
+
+
 def test_activations_above_4_gib(ops):
     """The wide kernels address activations with 32-bit byte offsets; a batch whose activations reach
     4 GiB must be kept away from them (and from every other 32-bit shortcut) by the launcher."""
