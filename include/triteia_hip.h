@@ -50,6 +50,13 @@ TRITEIA_HIP_API int triteia_hip_version(void);
 /* Text of the last error raised on this thread ("" if none). */
 TRITEIA_HIP_API const char* triteia_hip_last_error(void);
 
+/* The library's tuning knobs (environment variables TRITEIA_HIP_*, for tests and
+ * measurements) are read once, at the first call into the library; this reads
+ * them again.  Not to be called while another thread is inside the library, nor
+ * between triteia_hip_route_plan and the calls that consume its plan (both sides
+ * derive the plan's tile size from the knobs).  No counterpart in the reference. */
+TRITEIA_HIP_API void triteia_hip_reload_env(void);
+
 /* C = A @ dequant(B, meta, s) for one weight matrix.
  * Replaces marlin_cuda_2_4 (triteia/csrc/ops/marlin_nm.cu:42-46), bound by the
  * reference as mul_2_4 (triteia/csrc/ops/ops.cpp:88-116).
@@ -79,14 +86,25 @@ TRITEIA_HIP_API int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, con
 /* Run-list form: for run r < prob_r, rows starts[r] .. starts[r]+counts[r]-1 of
  * C = same rows of A @ dequant(B[indices[r]]).  indices / starts / counts are
  * int32 device arrays.  Replaces triteia_cuda_sbmm_2_4
- * (triteia/csrc/ops/triteia_nm_sbmm.cu:809-815), bound as sbmm_2_4 and, for the
- * host-loop variant, sbmm_forloop (triteia/csrc/ops/ops.cpp:279-327).
- * Rows not covered by a run are left untouched; runs with indices[r] outside
- * [0, n_deltas) are skipped.  n_deltas = number of matrices in B. */
+ * (triteia/csrc/ops/triteia_nm_sbmm.cu:809-815; the argument list is the same),
+ * bound as sbmm_2_4 and, for the host-loop variant, sbmm_forloop
+ * (triteia/csrc/ops/ops.cpp:279-327).  Rows not covered by a run are left
+ * untouched; runs with a negative index are skipped.  Like the reference's, this
+ * argument list does not say how many matrices B holds: every non-negative
+ * index must be valid. */
 TRITEIA_HIP_API int triteia_hip_sbmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, const void* indices,
                          const void* starts, const void* counts, int prob_m, int prob_n, int prob_k, int prob_r,
-                         int n_deltas, void* workspace, int groupsize, int dev, void* stream, int thread_k,
-                         int thread_m, int sms, int max_par);
+                         void* workspace, int groupsize, int dev, void* stream, int thread_k, int thread_m, int sms,
+                         int max_par);
+
+/* The same with a trailing n_deltas = number of matrices in B: runs whose index
+ * lies outside [0, n_deltas) are skipped instead of read out of bounds.  No
+ * counterpart in the reference (whose kernel trusts the indices,
+ * triteia_nm_sbmm.cu:743-748). */
+TRITEIA_HIP_API int triteia_hip_sbmm_2_4_bounded(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                 const void* indices, const void* starts, const void* counts, int prob_m, int prob_n,
+                                 int prob_k, int prob_r, void* workspace, int groupsize, int dev, void* stream,
+                                 int thread_k, int thread_m, int sms, int max_par, int n_deltas);
 
 /* Per-token routed form (no counterpart kernel in the reference; it replaces the
  * host-side routing prep of triteia/python/ops/matmul/sbmm.py:94-123 plus the

@@ -38,3 +38,20 @@ def check_close(got, ref, tol=2e-3, what=""):
     assert fro <= tol, f"{what}: relative Frobenius error {fro:.3e} > {tol}"
     assert mab <= tol, f"{what}: mean-abs error ratio {mab:.3e} > {tol}"
     return fro
+
+
+def reload_knobs():
+    """The library reads its TRITEIA_HIP_* knobs once; after a change of the environment it is told to read them again."""
+    from triteia_amd.python.capi import _ffi
+    _ffi.reload_env()
+
+
+def setknob(monkeypatch, name, value):
+    """Set one TRITEIA_HIP_* knob for the rest of the test (conftest restores the library's view afterwards)."""
+    monkeypatch.setenv(name, str(value))
+    reload_knobs()
+
+
+def delknob(monkeypatch, name):
+    monkeypatch.delenv(name, raising=False)
+    reload_knobs()

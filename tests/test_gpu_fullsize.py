@@ -16,6 +16,7 @@ import numpy as np
 import pytest
 import torch
 
+from tests.helpers import reload_knobs, setknob
 from triteia_amd import workloads as W
 
 pytestmark = pytest.mark.gpu
@@ -50,11 +51,13 @@ def _check_properties(ops, q, me, s, x, idx_np, sample_rows, sample_deltas, what
     # in its own order: the row-by-row comparison with a row routed on its own (always the K-split kernel) is made
     # on the K-split kernel's result for the batch, and the default result is held against that one.
     os.environ["TRITEIA_HIP_MID"] = "0"
+    reload_knobs()
     try:
         out_ksplit = ops.sbmm_4bit_2_4_native(q, x, me, s, idx)
         torch.cuda.synchronize()
     finally:
         del os.environ["TRITEIA_HIP_MID"]
+        reload_knobs()
     assert float((out.float() - out_ksplit.float()).norm()) <= 1e-3 * float(out_ksplit.float().norm()), what
     assert bool((out_ksplit[idx < 0] == 0).all())
     batch = out
@@ -180,7 +183,7 @@ def test_uniform_launches_of_one_workgroup_per_cu(ops, monkeypatch, b, t, k, m):
     for i in range(b):
         ref = x[i].float() @ unpack_2_4(q[i], me[i], s[i]).float()
         assert float((out[i].float() - ref).norm() / ref.norm()) <= 2e-3
-    monkeypatch.setenv("TRITEIA_HIP_WIDE", "0")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE", "0")
     narrow = ops.bmm_4bit_2_4(q, x, me, s)
     torch.cuda.synchronize()
     assert float((out.float() - narrow.float()).norm() / narrow.float().norm()) < 1e-4

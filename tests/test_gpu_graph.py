@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import triteia_oracle as orc
-from tests.helpers import activations, check_close, make_deltas, to_gpu
+from tests.helpers import activations, check_close, make_deltas, setknob, to_gpu
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -33,7 +33,7 @@ def _capture(fn):
 def test_routed_sbmm_replays(monkeypatch, T, N, k, m, seed):
     from triteia_amd.python.capi import routed_workspace, sbmm_2_4_routed
     # the wide kernel takes its tiles however few they are (by default only when they fill the chip)
-    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
     print(f"[case] graph replay of routed sbmm T={T} N={N} k={k} m={m} seed={seed}", flush=True)
     qw, meta, s = make_deltas(N, k, m, seed)
     gq, gm, gs = to_gpu(qw, meta, s)

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from oracle import triteia_oracle as orc
-from tests.helpers import activations, check_close, make_deltas, to_gpu
+from tests.helpers import activations, check_close, delknob, make_deltas, reload_knobs, setknob, to_gpu
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -24,9 +24,9 @@ WIDE_MIN_BATCH = 512          # in these tests plans carry wide tiles from this 
 
 @pytest.fixture(autouse=True)
 def _wide_tiles_from_512_tokens(monkeypatch):
-    monkeypatch.setenv("TRITEIA_HIP_WIDE_MIN_BATCH", str(WIDE_MIN_BATCH))
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE_MIN_BATCH", str(WIDE_MIN_BATCH))
     # ... and the wide kernel takes them however few they are (by default only when they fill the chip)
-    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
 
 
 def say(msg):
@@ -61,7 +61,7 @@ def test_matmul_4bit_2_4(ops, n, k, m, seed):
     check_close(out, ref, what="matmul_4bit_2_4")
 
 
-@pytest.mark.parametrize("kernel", ["wide64", "wide64ks", "wide128", "wide32", "wide32ks"])
+@pytest.mark.parametrize("kernel", ["wide64", "wide64ks", "tile256", "wide32", "wide32ks"])
 @pytest.mark.parametrize("n,k,m,seed", [
     (64, 128, 512, 21), (128, 128, 512, 22), (128, 256, 128, 23),      # one tile, 1 and 2 k steps
     (200, 384, 384, 24), (321, 512, 640, 25), (130, 640, 256, 26),     # ragged tokens, partial column groups
@@ -72,16 +72,15 @@ def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
     """The matrix-core-bound kernels (64- and 128-token tiles) and the 32-token build with two steps of
     weights in flight, forced onto small ragged shapes that the launcher would give to the narrow kernel."""
     say(f"matmul {kernel} n={n} k={k} m={m} seed={seed}")
-    monkeypatch.setenv("TRITEIA_HIP_WIDE_MIN_UNITS", "1")
-    monkeypatch.setenv("TRITEIA_HIP_WIDE128_MIN_UNITS", "1")
-    monkeypatch.setenv("TRITEIA_HIP_WIDE128_MIN_K", "0")
-    monkeypatch.setenv("TRITEIA_HIP_WIDE128", "1" if kernel == "wide128" else "0")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE_MIN_UNITS", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_TILE256_MIN_UNITS", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_TILE256", "1" if kernel == "tile256" else "0")
     if kernel in ("wide32", "wide32ks"):   # takes the tokens ahead of the other two whenever its window of units is open
-        monkeypatch.setenv("TRITEIA_HIP_WIDE32_MIN_UNITS", "1")
-        monkeypatch.setenv("TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")
+        setknob(monkeypatch, "TRITEIA_HIP_WIDE32_MIN_UNITS", "1")
+        setknob(monkeypatch, "TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")
     # wide32ks: eight wavefronts per workgroup, each half of them on half of the k steps
-    monkeypatch.setenv("TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS", "1000000000" if kernel == "wide32ks" else "0")
-    monkeypatch.setenv("TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS", "1000000000" if kernel == "wide64ks" else "0")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS", "1000000000" if kernel == "wide32ks" else "0")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS", "1000000000" if kernel == "wide64ks" else "0")
     qw, meta, s = make_deltas(1, k, m, seed)
     x = activations(n, k, seed + 1)
     ref = orc.matmul_4bit_2_4(qw[0], x, meta[0], s[0])
@@ -90,7 +89,7 @@ def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
     torch.cuda.synchronize()
     check_close(out, ref, what=f"matmul_4bit_2_4 {kernel}")
     # same inputs through the narrow kernel: equal up to the order of fp32 accumulation
-    monkeypatch.setenv("TRITEIA_HIP_WIDE", "0")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE", "0")
     narrow = ops.matmul_4bit_2_4(gq, gx, gm, gs)
     torch.cuda.synchronize()
     rel = ((out.float() - narrow.float()).norm() / narrow.float().norm()).item()
@@ -181,15 +180,15 @@ def test_bmm_4bit_2_4(ops, b, t, k, m, seed):
 def test_bmm_32_token_wide_kernel(ops, monkeypatch, b, t, k, m, seed):
     """Uniform groups on the 32-token build of the wide kernel (by default only for launches of 160 to 448 units)."""
     say(f"bmm on 32-token wide tiles b={b} t={t} k={k} m={m} seed={seed}")
-    monkeypatch.setenv("TRITEIA_HIP_WIDE32_MIN_UNITS", "1")
-    monkeypatch.setenv("TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE32_MIN_UNITS", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")
     qw, meta, s = make_deltas(b, k, m, seed)
     x = activations(b * t, k, seed + 1).reshape(b, t, k)
     gq, gm, gs, gx = to_gpu(qw, meta, s, x)
     out = ops.bmm_4bit_2_4(gq, gx, gm, gs)
     torch.cuda.synchronize()
     check_close(out, orc.bmm_4bit_2_4(qw, x, meta, s), what="bmm on 32-token wide tiles")
-    monkeypatch.setenv("TRITEIA_HIP_WIDE", "0")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE", "0")
     narrow = ops.bmm_4bit_2_4(gq, gx, gm, gs)
     torch.cuda.synchronize()
     assert float((out.float() - narrow.float()).norm() / narrow.float().norm()) < 1e-4
@@ -297,9 +296,9 @@ def test_routing_is_bit_exact_on_exact_arithmetic(ops, monkeypatch, T, N, k, m, 
     assert torch.equal(ops.sbmm_4bit_2_4_native(gq, gx, gm, gs, gi), want)
     # a plan with wide tiles also carries a narrow-only cut of the same tokens; the kernels choose on the
     # device (here: a bar no launch reaches, so the narrow-only cut runs and the wide launch returns at once)
-    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1000000000")
+    setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1000000000")
     assert torch.equal(ops.sbmm_4bit_2_4_native(gq, gx, gm, gs, gi), want)
-    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
     assert torch.equal(ops.sbmm_4bit_2_4_forloop(gq, gx, gm, gs, gi), want)
     order = np.argsort(idx, kind="stable")
     gxs, gis = to_gpu(x[order], idx[order])
@@ -343,6 +342,7 @@ def test_fused_routing_static_groups(ops, monkeypatch, T, N, used, seed):
             monkeypatch.delenv(key, raising=False)
         for key, value in env.items():
             monkeypatch.setenv(key, value)
+        reload_knobs()
         out = torch.full((T, m), 3.0, dtype=torch.float16, device=DEV)      # rows without a delta must stay as they are
         from triteia_amd.python.capi import sbmm_2_4_routed
         sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
@@ -405,11 +405,11 @@ def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, 
     gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
     outs = []
     for passes in ("4", "2", "1", None):
-        monkeypatch.setenv("TRITEIA_HIP_FUSED_ROUTE", "0")
+        setknob(monkeypatch, "TRITEIA_HIP_FUSED_ROUTE", "0")
         if passes is None:
-            monkeypatch.delenv("TRITEIA_HIP_PASS_NT", raising=False)
+            delknob(monkeypatch, "TRITEIA_HIP_PASS_NT")
         else:
-            monkeypatch.setenv("TRITEIA_HIP_PASS_NT", passes)
+            setknob(monkeypatch, "TRITEIA_HIP_PASS_NT", passes)
         out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
         sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
         torch.cuda.synchronize()
@@ -436,8 +436,8 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     untouched rows stay untouched; accumulation in place."""
     say(f"32-token wide kernel T={T} N={N} k={k} m={m} seed={seed} wide_bar={wide_bar}")
     from triteia_amd.python.capi import sbmm_2_4_routed
-    monkeypatch.setenv("TRITEIA_HIP_FUSED_ROUTE", "0")
-    monkeypatch.setenv("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", wide_bar)
+    setknob(monkeypatch, "TRITEIA_HIP_FUSED_ROUTE", "0")
+    setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", wide_bar)
     qw, meta, s = make_deltas(N, k, m, seed)
     x = activations(T, k, seed + 1)
     idx = np.random.default_rng(seed + 2).integers(-1, N, size=T).astype(np.int32)
@@ -447,9 +447,9 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
     outs = {}
     for mid in ("1", "0"):
-        monkeypatch.setenv("TRITEIA_HIP_MID", mid)
-        monkeypatch.setenv("TRITEIA_HIP_MID_MIN_UNITS", "1")
-        monkeypatch.setenv("TRITEIA_HIP_MID_MIN_COLUMN_GROUPS", "1")
+        setknob(monkeypatch, "TRITEIA_HIP_MID", mid)
+        setknob(monkeypatch, "TRITEIA_HIP_MID_MIN_UNITS", "1")
+        setknob(monkeypatch, "TRITEIA_HIP_MID_MIN_COLUMN_GROUPS", "1")
         out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
         sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
         torch.cuda.synchronize()
@@ -461,7 +461,7 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     assert not torch.equal(outs["1"], outs["0"]) or k <= 128, "the knob did not change the kernel"
     assert float((outs["1"].float() - outs["0"].float()).norm()) <= 1e-3 * float(outs["0"].float().norm())
     # accumulate in place on top of a base
-    monkeypatch.setenv("TRITEIA_HIP_MID", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_MID", "1")
     base = torch.from_numpy(activations(T, m, seed + 3)).to(DEV)
     acc = base.clone()
     sbmm_2_4_routed(gx, gq, gm, acc, gs, gi, accumulate=True)

@@ -24,9 +24,26 @@ HIPCC_FLAGS = [
 ]
 
 
+# The wide kernels wait for their direct-to-LDS loads with hand-counted `s_waitcnt vmcnt(N)`: N counts
+# the loads the compiler emits behind them in program order.  The counts were checked against the assembly
+# output of this compiler; another one may order or split the loads differently, so the build refuses it
+# unless TRITEIA_HIP_ANY_COMPILER=1 says that the counts have been checked again (`-S`, then the GPU parity tests).
+VERIFIED_COMPILER = "roc-7.2.0"
+
+
+def check_compiler(hipcc: str) -> str:
+    out = subprocess.run([hipcc, "--version"], capture_output=True, text=True).stdout
+    if VERIFIED_COMPILER not in out and os.environ.get("TRITEIA_HIP_ANY_COMPILER") != "1":
+        raise RuntimeError(
+            f"{hipcc} is not the compiler the hand-counted waits were verified with ({VERIFIED_COMPILER}):\n{out}"
+            "set TRITEIA_HIP_ANY_COMPILER=1 after checking them again")
+    return out
+
+
 def build(verbose: bool = True, extra_flags=()) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    check_compiler(hipcc)
     cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-o", LIB, SRC]
     if verbose:
         print("[triteia_amd.build]", " ".join(cmd), flush=True)

@@ -99,9 +99,6 @@ struct Sparse24Args {
   int raw_static;           // fused routing with group g = delta g: weights are requested before the indices arrive
   int rot_spread;           // steps between the starting points of consecutive deltas' walks over K (0: all start at step 0)
   int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run
-#ifdef TRITEIA_HIP_TIMELINE
-  long long* timeline;      // [unit][wave][4] 100 MHz timestamps (debug builds only)
-#endif
 };
 
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
@@ -181,9 +178,6 @@ struct TileCtx {
   // the parts in order.
   int raw_list[kRawParts];
   int raw_before[kRawParts + 1];
-#ifdef TRITEIA_HIP_TIMELINE
-  long long ts[4];          // debug builds: entry, operands requested, K loop done, end
-#endif
 };
 
 // One pass over K for up to 16*NTT tokens of one group: loads, sparse MFMAs, cross-wave
@@ -337,9 +331,6 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   // registers (ring of fragments, statically indexed through the unrolled inner loop).
   // The body is branch-free apart from the wave-uniform "is this step real" test around the
   // arithmetic, so each iteration issues the same loads and waits for exactly its own.
-#ifdef TRITEIA_HIP_TIMELINE
-  c.ts[1] = wall_clock64();
-#endif
 #pragma unroll
   for (int j = 0; j < DEPTH; j++) load_x(ring[j], wave + j * KW);
   for (int st = wave; st < n_steps; st += DEPTH * KW) {
@@ -352,9 +343,6 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
     }
   }
 
-#ifdef TRITEIA_HIP_TIMELINE
-  c.ts[2] = wall_clock64();
-#endif
   // cross-wave reduction + epilogue, one 16-token tile at a time
 #pragma unroll
   for (int nt = 0; nt < NTT; nt++) {
@@ -409,9 +397,6 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   __shared__ float red[KW][16][kRedStride];
   __shared__ int s_rows[16 * NT];
 
-#ifdef TRITEIA_HIP_TIMELINE
-  const long long ts_entry = wall_clock64();
-#endif
   // Unit = (group, column block).  Workgroups are dealt round-robin to the 8 XCDs (each with
   // its own L2); the column blocks of a group are numbered so that every XCD owns a contiguous
   // run of them: the per-group unit count is padded to a multiple of 8 (padding units exit).
@@ -575,12 +560,6 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
     // the next pass over this group's tokens reuses s_rows / red
     if (t0 + gridDim.y * 16 * NT < count) lds_barrier();
   }
-#ifdef TRITEIA_HIP_TIMELINE
-  if (p.timeline && c.lane == 0 && blockIdx.y == 0) {
-    long long* t = p.timeline + ((long)unit * KW + c.wave) * 4;
-    t[0] = ts_entry; t[1] = c.ts[1]; t[2] = c.ts[2]; t[3] = wall_clock64();
-  }
-#endif
 }
 
 }  // namespace triteia_hip

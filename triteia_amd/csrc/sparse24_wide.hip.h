@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   // counts a direct-to-LDS load as an LDS write, which the release fence of every barrier and
   // the first LDS read behind it must complete, i.e. it drains every outstanding request (the
   // weights requested a moment ago included) once per K step.  The LDS address of a request is
-  // M0 + 16 * lane.
+  // M0 + 16 * lane; M0 is an input operand of the statement, so the compiler writes it and knows it is live.
   const uint32_t lds_x_wave = (uint32_t)(uintptr_t)&xs[kh][0][4 * wave][0];
   auto issue_x = [&](int st) {
     const int stc = min(step0 + min(st, n_steps - 1), all_steps - 1);   // past the end: refetch a valid tile (never read)
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
     for (int ii = 0; ii < NT; ii++) {
       const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_x_wave + (stage * TOK + 16 * ii) * 256);
       const _Float16* base = p.x + stc * 128;
-      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(xoff[ii]), "s"(base), "s"(dst) : "memory");
+      asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(xoff[ii]), "s"(base), "{m0}"(dst) : "memory");
     }
   };
 

@@ -8,12 +8,12 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "lora.hip.h"
 #include "route_plan.hip.h"
 #include "sparse24_gemm.hip.h"
 #include "sparse24_wide.hip.h"
-#include "sparse24_wide128.hip.h"
 
 namespace {
 
@@ -46,10 +46,51 @@ int check_launch(const char* what) {
   return TRITEIA_HIP_OK;
 }
 
-int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return v && *v ? atoi(v) : dflt;
+// Tuning knobs.  Each can be set through an environment variable of the same name in capitals with the
+// prefix TRITEIA_HIP_ (for tests and measurements); the variables are read ONCE, at the first call into the
+// library, and again only when triteia_hip_reload_env() is called: an ordinary call does no getenv.
+// kUnset marks knobs whose default depends on the launch.
+constexpr int kUnset = -0x7fffffff;
+struct Knobs {
+  int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, pass_nt = 0;
+  int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
+  int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
+  int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset;
+  int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
+  int tile256 = 1, tile256_min_units = kUnset, ksplit = 1;
+};
+Knobs g_knobs;
+std::once_flag g_knobs_once;
+
+void read_knobs() {
+  Knobs k;
+  struct { const char* name; int* dst; } table[] = {
+      {"NT", &k.nt}, {"KW", &k.kw}, {"DEPTH", &k.depth}, {"ROT_SPREAD", &k.rot_spread}, {"XCD_SWIZZLE", &k.xcd_swizzle},
+      {"PASS_NT", &k.pass_nt}, {"WIDE", &k.wide}, {"WIDE_DEPTH", &k.wide_depth}, {"WIDE_MIN_UNITS", &k.wide_min_units},
+      {"WIDE_MIN_BATCH", &k.wide_min_batch}, {"PLAN_WIDE_MIN_UNITS", &k.plan_wide_min_units},
+      {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
+      {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
+      {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
+      {"MID_MIN_UNITS", &k.mid_min_units}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
+      {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units},
+      {"KSPLIT", &k.ksplit},
+  };
+  char name[64];
+  for (auto& e : table) {
+    snprintf(name, sizeof(name), "TRITEIA_HIP_%s", e.name);
+    const char* v = getenv(name);
+    if (v && *v) *e.dst = atoi(v);
+  }
+  g_knobs = k;
 }
+
+const Knobs& knobs() {
+  std::call_once(g_knobs_once, read_knobs);
+  return g_knobs;
+}
+
+// value of a knob whose default depends on the launch
+inline int knob_or(int v, long dflt) { return v == kUnset ? (int)dflt : v; }
 
 int check_gemm_shape(int prob_m, int prob_n, int prob_k, int groupsize) {
   if (groupsize != -1)
@@ -62,7 +103,7 @@ int check_gemm_shape(int prob_m, int prob_n, int prob_k, int groupsize) {
 // Token tile of the grouped kernel: 16 * NT rows share one pass over the weights.  Chosen from
 // what the host knows (tokens, groups); the routing plan cuts groups into tiles of this size.
 int pick_nt(long tokens, long groups) {
-  const int forced = env_int("TRITEIA_HIP_NT", 0);
+  const int forced = knobs().nt;
   if (forced == 1 || forced == 2 || forced == 4) return forced;
   if (groups < 1) groups = 1;
   if (tokens <= 16) return 1;
@@ -78,7 +119,7 @@ int pick_nt(long tokens, long groups) {
 // one workgroup per CU, else 16-token tiles with the tokens split across workgroups (measured on
 // one 4096 x 4096 matrix: 64 tokens 24.4 -> 12.2 us, 128 tokens 24.2 -> 12.4 us, 256 tokens 24.4 -> 19.1 us).
 int pick_nt_uniform(long tokens, long groups, long col_blocks) {
-  const int forced = env_int("TRITEIA_HIP_NT", 0);
+  const int forced = knobs().nt;
   if (forced == 1 || forced == 2 || forced == 4) return forced;
   for (int nt = 4; nt >= 2; nt /= 2) {
     if (tokens <= 8 * nt) continue;   // a narrower tile holds them all
@@ -106,7 +147,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   // fp32 sums, and a routed token must have the same bits whatever the size of its batch.
   const bool uniform = !a.raw_indices && !a.tiles && !a.g_delta;
   const bool one_per_cu = uniform && (nt == 1 || nt == 2) && (long)a.n_groups * cb_pad * tsplit <= 256;
-  const int kw = env_int("TRITEIA_HIP_KW", one_per_cu ? 8 : 4);
+  const int kw = knob_or(knobs().kw, one_per_cu ? 8 : 4);
   // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight (2 with
   // two), the 32-token kernel 2 per CU with two, the 64-token kernel 1 per CU with one.  Fused
   // routing in its eager form keeps one step in flight (measured: a second step requested ahead of
@@ -116,7 +157,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   // of each wave's chain of requests rather than by bandwidth: a second step in flight pays there
   // (5-12 % measured) while it costs time on full launches
   const bool small = (long)a.n_groups * cb_pad * tsplit <= 512;
-  const int depth = env_int("TRITEIA_HIP_DEPTH", eager || kw == 8 ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1));
+  const int depth = knob_or(knobs().depth, eager || kw == 8 ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1));
   if (eager && !(kw == 4 && ((nt == 1 && depth == 2) || (nt == 1 && depth == 1) || (nt == 2 && depth == 1) || (nt == 4 && depth == 1)))) {
     a.raw_static = 0;   // no eager build of this variant: route first, then request
     a.n_groups = a.raw_count < a.n_deltas ? a.raw_count : a.n_deltas;
@@ -128,7 +169,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
     const long side_by_side = 512 / cb_pad;
     const int n_steps = (a.k / 32 + 3) / 4;
     const long spread = side_by_side >= 4 ? n_steps / (side_by_side < 16 ? side_by_side : 16) : 0;
-    a.rot_spread = env_int("TRITEIA_HIP_ROT_SPREAD", (int)spread);
+    a.rot_spread = knob_or(knobs().rot_spread, spread);
   }
   const long units = (long)a.n_groups * cb_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
@@ -162,10 +203,7 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.m = prob_m;
   a.k = prob_k;
   a.n_deltas = n_deltas;
-  a.xcd_swizzle = env_int("TRITEIA_HIP_XCD_SWIZZLE", 1);
-#ifdef TRITEIA_HIP_TIMELINE
-  a.timeline = reinterpret_cast<long long*>(strtoull(getenv("TRITEIA_HIP_TIMELINE_PTR") ? getenv("TRITEIA_HIP_TIMELINE_PTR") : "0", nullptr, 0));
-#endif
+  a.xcd_swizzle = knobs().xcd_swizzle;
 }
 
 
@@ -186,53 +224,28 @@ int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   Sparse24Args b = a;
   if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
-  if (tok == 32 && units <= env_int("TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS", kWide32KSplitMaxUnits))
+  if (tok == 32 && units <= knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits))
     hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false, 2>), dim3((unsigned)units), dim3(512), 0, st, b);
   else if (tok == 32)
     hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false>), dim3((unsigned)units), dim3(256), 0, st, b);
-  else if (units <= env_int("TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS", kWide64KSplitMaxUnits) &&
+  else if (units <= knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits) &&
            !a.tiles)   // (a plan's launch is sized by an upper bound on its tiles; at 190-230 real units it measured the same either way)
     hipLaunchKernelGGL((sparse24_wide_kernel<1, kWideTokens, false, 2>), dim3((unsigned)units), dim3(512), 0, st, b);
-  else if (env_int("TRITEIA_HIP_WIDE_DEPTH", 1) == 1)
+  else if (knobs().wide_depth == 1)
     hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3((unsigned)units), dim3(256), 0, st, b);
   else
     hipLaunchKernelGGL((sparse24_wide_kernel<2>), dim3((unsigned)units), dim3(256), 0, st, b);
   return check_launch("sparse24_wide_kernel");
 }
 
-// 128-token x 512-column tiles (one workgroup per CU, 128.5 KB of dynamic LDS).
-int launch_wide128(const Sparse24Args& a, hipStream_t st) {
-  if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
-  const long cgs = (a.m / 128 + 3) / 4;
-  const long cg_pad = (cgs + 7) / 8 * 8;
-  const long chunks = a.tiles ? 1 : (a.uniform_count + kWide128Tokens - 1) / kWide128Tokens;
-  const long units = (long)a.n_groups * chunks * cg_pad;
-  if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
-  // the attribute is per device; setting it again is cheap and keeps the library free of global state
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse24_wide128_kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kWide128LdsBytes) != hipSuccess)
-    return fail(TRITEIA_HIP_ERR_RUNTIME, "sparse24_wide128_kernel: cannot reserve %d bytes of LDS", kWide128LdsBytes);
-  Sparse24Args b = a;
-  if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
-  hipLaunchKernelGGL(sparse24_wide128_kernel, dim3((unsigned)units), dim3(256), kWide128LdsBytes, st, b);
-  return check_launch("sparse24_wide128_kernel");
-}
-
-// The wide kernels pay off when there are enough tiles to occupy the GPU; below that the
-// narrow kernel's smaller units win.  TRITEIA_HIP_WIDE=0 disables both; the 128-token one is off unless
-// TRITEIA_HIP_WIDE128=1 (since the 64-token kernel's requests stay in flight across its barriers it is
-// as fast or faster on every shape measured: 4096 tokens on 8192 x 8192 279-296 us against 286-301 us, on
-// 8192 x 28672 970 us both, 1024 tokens there 258 against 270 us);
-// TRITEIA_HIP_WIDE_MIN_UNITS / TRITEIA_HIP_WIDE128_MIN_UNITS move the thresholds.
-bool wide_enabled() { return env_int("TRITEIA_HIP_WIDE", 1) != 0; }
-bool wide128_enabled() { return wide_enabled() && env_int("TRITEIA_HIP_WIDE128", 0) != 0; }
+// The wide kernel pays off when there are enough tiles to occupy the GPU; below that the narrow
+// kernel's smaller units win.  Knob `wide` = 0 disables it; `wide_min_units` moves the threshold.
+bool wide_enabled() { return knobs().wide != 0; }
 constexpr long kWideMinUnits = 160;   // 4096 x 4096: 1024 tokens (128 tiles) 54.9 us wide against 46.5 us narrow, 1536 tokens (192) 60.8 against 71.1
-constexpr long kWide128MinUnits = 192;
 constexpr long kWide32MinUnits = 160, kWide32MaxUnits = 448;   // (32-token tile, 512-column group) units: see launch_uniform
 
 // `tokens` rows per group, `stride` rows between groups: the head of each group goes to the
-// 128-token kernel, then to the 64-token kernel (full tiles, and a rest above half a tile),
-// what is left to the narrow one.
+// 64-token kernel (full tiles, and a rest above half a tile), what is left to the narrow one.
 int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n_groups, hipStream_t st) {
   a.n_groups = n_groups;
   a.uniform_stride = stride;
@@ -261,33 +274,22 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
     // 50.8 -> 46.0 us; 4096 x 11008 with 384 / 640 tokens 47.2 -> 43.0, 51.4 -> 46.0 us; 8192 x 8192 with 768 tokens 88.7 ->
     // 72.5 us; 8192 x 28672 with 192 tokens 89.4 -> 73.0 us)
     ks64 = wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= kWideTokens &&
-           units32 > env_int("TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS", kWide32KSplitMaxUnits) &&
+           units32 > knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits) &&
            (long)n_groups * ((tokens + kWideTokens - 1) / kWideTokens) * ((cgs + 7) / 8 * 8) <=
-               env_int("TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS", kWide64KSplitMaxUnits);
+               knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits);
     if (!ks64 && wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= 32 &&
-        units32 >= env_int("TRITEIA_HIP_WIDE32_MIN_UNITS", kWide32MinUnits) &&
-        units32 <= env_int("TRITEIA_HIP_WIDE32_MAX_UNITS", kWide32MaxUnits)) {
+        units32 >= knob_or(knobs().wide32_min_units, kWide32MinUnits) &&
+        units32 <= knob_or(knobs().wide32_max_units, kWide32MaxUnits)) {
       a.uniform_first = 0;
       a.uniform_count = tokens;
       if (int e = launch_wide(a, st, 32)) return e;
       done = tokens;
     }
   }
-  // (the 128-token kernel pays from k = 8192 on: 2-3 % faster than the 64-token kernel at 8192 x 8192 and
-  // 8192 x 28672, 4-8 % slower at 4096 x 4096 and 4096 x 11008, whose K loops are too short for its pipeline)
-  if (done == 0 && wide128_enabled() && a.k % 128 == 0 && a.k >= env_int("TRITEIA_HIP_WIDE128_MIN_K", 8192) && x_below_4g &&
-      (long)n_groups * (tokens / kWide128Tokens) * cgs >= env_int("TRITEIA_HIP_WIDE128_MIN_UNITS", kWide128MinUnits)) {
-    int t = tokens / kWide128Tokens * kWide128Tokens;
-    if (tokens - t > kWideTokens) t = tokens;
-    a.uniform_first = 0;
-    a.uniform_count = t;
-    if (int e = launch_wide128(a, st)) return e;
-    done = t;
-  }
   int rest = tokens - done;
   if (rest > 0 && wide_enabled() && a.k % 128 == 0 && x_below_4g &&
       (done > 0 ? rest >= kPlanWideMinRest
-                : ks64 || (long)n_groups * (rest / kWideTokens) * cgs >= env_int("TRITEIA_HIP_WIDE_MIN_UNITS", kWideMinUnits))) {
+                : ks64 || (long)n_groups * (rest / kWideTokens) * cgs >= knob_or(knobs().wide_min_units, kWideMinUnits))) {
     int t = rest / kWideTokens * kWideTokens;
     // A rest above half a tile becomes a tile of its own; a smaller one too while the launch stays within one
     // round of workgroups (two per CU), where its workgroups cost nothing and a launch of the narrow kernel for them
@@ -314,7 +316,12 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
 
 extern "C" {
 
-int triteia_hip_version(void) { return 1000; }
+int triteia_hip_version(void) { return 1001; }
+
+void triteia_hip_reload_env(void) {
+  knobs();        // (so that a first call later on does not overwrite what is read here)
+  read_knobs();
+}
 
 const char* triteia_hip_last_error(void) { return g_err; }
 
@@ -353,10 +360,10 @@ int triteia_hip_bmm_2_4(const void* A, const void* B, const void* meta, void* C,
   return triteia_hip_bmm_2_4_tokens(A, B, meta, C, s, prob_m, prob_n, 1, prob_k, dev, stream);
 }
 
-int triteia_hip_sbmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, const void* indices,
-                         const void* starts, const void* counts, int prob_m, int prob_n, int prob_k, int prob_r,
-                         int n_deltas, void* workspace, int groupsize, int dev, void* stream, int thread_k,
-                         int thread_m, int sms, int max_par) {
+int triteia_hip_sbmm_2_4_bounded(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                 const void* indices, const void* starts, const void* counts, int prob_m, int prob_n,
+                                 int prob_k, int prob_r, void* workspace, int groupsize, int dev, void* stream,
+                                 int thread_k, int thread_m, int sms, int max_par, int n_deltas) {
   (void)workspace; (void)thread_k; (void)thread_m; (void)sms; (void)max_par;
   if (int e = check_gemm_shape(prob_m, prob_n, prob_k, groupsize)) return e;
   if (prob_r < 0 || n_deltas < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sbmm_2_4: runs=%d deltas=%d", prob_r, n_deltas);
@@ -376,6 +383,15 @@ int triteia_hip_sbmm_2_4(const void* A, const void* B, const void* meta, void* C
   long tsplit = (4L * prob_n / prob_r + 16 * nt - 1) / (16 * nt);
   if (tsplit > 16) tsplit = 16;
   return launch_sparse24(a, nt, tsplit, static_cast<hipStream_t>(stream));
+}
+
+int triteia_hip_sbmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, const void* indices,
+                         const void* starts, const void* counts, int prob_m, int prob_n, int prob_k, int prob_r,
+                         void* workspace, int groupsize, int dev, void* stream, int thread_k, int thread_m, int sms,
+                         int max_par) {
+  // the reference's argument list carries no number of matrices: every non-negative index is taken as valid
+  return triteia_hip_sbmm_2_4_bounded(A, B, meta, C, s, indices, starts, counts, prob_m, prob_n, prob_k, prob_r, workspace,
+                                      groupsize, dev, stream, thread_k, thread_m, sms, max_par, 0x7fffffff);
 }
 
 size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n_deltas) {
@@ -407,8 +423,8 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   const int tile = triteia_hip_plan_tile_tokens(prob_n, n_deltas);
   // (64-token plans as well, on the 64-token build, where K is short: cfg3 at 1024 / 2048 tokens 196 -> 170 /
   // 250 -> 214 us; at k = 8192 the narrow kernel's workgroups live long enough: cfg4 at 2048 tokens 1478 -> 1523 us)
-  const bool mid64 = tile == 64 && env_int("TRITEIA_HIP_MID64", 1) && prob_k < env_int("TRITEIA_HIP_MID64_MAX_K", 8192);
-  if (!env_int("TRITEIA_HIP_MID", 1) || (tile != 32 && !mid64)) return false;
+  const bool mid64 = tile == 64 && knobs().mid64 && prob_k < knobs().mid64_max_k;
+  if (!knobs().mid || (tile != 32 && !mid64)) return false;
   if (prob_k % 128 != 0 || (long)prob_n * prob_k * 2 >= (1L << 32)) return false;   // whole K steps, 32-bit activation offsets
   const long tiles = (n_deltas < prob_n ? n_deltas : prob_n) + prob_n / tile;
   // (and only with a few tokens per tile at least: with two or three the shared activation tile saves nothing
@@ -417,13 +433,13 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   // (and a layer of 16 column groups at least: on m = 4096 it is even at best, 64 deltas with 8 tokens each 80 us
   // both ways, and loses with few tokens per tile, 128 deltas with 6 each 146 -> 164 us)
   const long cgs = (prob_m / 128 + 3) / 4;
-  if (cgs < env_int("TRITEIA_HIP_MID_MIN_COLUMN_GROUPS", 16)) return false;
-  return tiles * cgs >= env_int("TRITEIA_HIP_MID_MIN_UNITS", kMidMinUnits);
+  if (cgs < knobs().mid_min_column_groups) return false;
+  return tiles * cgs >= knob_or(knobs().mid_min_units, kMidMinUnits);
 }
 constexpr int kFusedMaxTokens = 64 * kRawParts;   // kRawParts tokens per lane of a wavefront
 static int plan_has_wide(int prob_n, int n_deltas) {
   const long groups = n_deltas < prob_n ? n_deltas : prob_n;
-  return wide_enabled() && prob_n >= env_int("TRITEIA_HIP_WIDE_MIN_BATCH", 256) && prob_n >= 8 * groups;
+  return wide_enabled() && prob_n >= knobs().wide_min_batch && prob_n >= 8 * groups;
 }
 
 int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
@@ -476,7 +492,7 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
   if (wide) {
     a.tiles_alt = reinterpret_cast<const int4*>(ws + L.all);
     a.wide_gate = (prob_m / 128 + 3) / 4;
-    a.wide_min_units = env_int("TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", kPlanWideMinUnits);
+    a.wide_min_units = knob_or(knobs().plan_wide_min_units, kPlanWideMinUnits);
     // The wide kernel needs whole 128-deep K steps, and a batch that could not reach the bar
     // even with most of its tokens in wide tiles (one per 48 tokens) is not worth the empty
     // launch: then the bar is out of reach on the device too and every tile list is the narrow-only one.
@@ -498,7 +514,7 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     const long cb_pad = (prob_m / 128 + 7) / 8 * 8;
     if ((long)a.n_groups * cb_pad < 200)
       while (pass_nt > 1 && (long)a.n_groups * cb_pad * (tile / (16 * pass_nt)) < 256) pass_nt /= 2;
-    const int forced = env_int("TRITEIA_HIP_PASS_NT", 0);
+    const int forced = knobs().pass_nt;
     if ((forced == 1 || forced == 2 || forced == 4) && 16 * forced <= tile) pass_nt = forced;
   }
   if (mid) {
@@ -539,9 +555,9 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   // plan pays from 128 tokens on whatever the number of deltas, the plan launch being small against the kernel
   // and the wide kernels taking hot deltas: 8 / 4 deltas of 8192 x 28672 with 128 / 256 tokens 145 -> 130 /
   // 160 -> 122 us, while 8 or 16 deltas of 4096 x 11008 stay 8-12 % faster routed inside the kernel)
-  const bool eager_ok = n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && env_int("TRITEIA_HIP_EAGER", 1);
-  if (prob_n <= env_int("TRITEIA_HIP_FUSED_MAX_TOKENS", kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
-      n_deltas <= (prob_n > 64 ? 32 : 64) && env_int("TRITEIA_HIP_FUSED_ROUTE", 1) &&
+  const bool eager_ok = n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && knobs().eager;
+  if (prob_n <= knob_or(knobs().fused_max_tokens, kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
+      n_deltas <= (prob_n > 64 ? 32 : 64) && knobs().fused_route &&
       !(prob_n >= 128 && ((!eager_ok && mid_tiles(prob_n, n_deltas, prob_m, prob_k)) || (long)prob_k * prob_m >= (1L << 27)))) {
     // small batch: the multiply kernel routes by itself, no plan, no workspace traffic
     if (!token_indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null indices");

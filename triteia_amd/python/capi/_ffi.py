@@ -25,7 +25,9 @@ SIGNATURES = {
     "triteia_hip_mul_2_4": (_c_int, [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
     "triteia_hip_bmm_2_4": (_c_int, [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
     "triteia_hip_bmm_2_4_tokens": (_c_int, [_c_vp] * 5 + [_c_int] * 4 + [_c_int, _c_vp]),
-    "triteia_hip_sbmm_2_4": (_c_int, [_c_vp] * 8 + [_c_int] * 5 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
+    "triteia_hip_reload_env": (None, []),
+    "triteia_hip_sbmm_2_4": (_c_int, [_c_vp] * 8 + [_c_int] * 4 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
+    "triteia_hip_sbmm_2_4_bounded": (_c_int, [_c_vp] * 8 + [_c_int] * 4 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 5),
     "triteia_hip_sbmm_2_4_routed": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_vp, _c_sz, _c_int, _c_int, _c_vp]),
     "triteia_hip_sbmm_2_4_planned": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_int, _c_vp]),
     "triteia_hip_sbmm_routed_workspace_bytes": (_c_sz, [_c_int, _c_int]),
@@ -57,6 +59,12 @@ def lib():
             fn.argtypes = args
         _lib = handle
     return _lib
+
+
+def reload_env() -> None:
+    """Make the library read its TRITEIA_HIP_* tuning knobs from the environment again (it reads
+    them once, at its first call)."""
+    lib().triteia_hip_reload_env()
 
 
 def last_error() -> str:

@@ -78,9 +78,17 @@ def bmm_2_4(A, B, meta, C, s, workspace, thread_k=-1, thread_m=-1, sms=-1, max_p
         _raise(_ffi.ERR_KERN_SHAPE, prob_m, batch, prob_k, thread_k, thread_m, groupsize)
     if prob_m % 128 == 0 and prob_k % 64 == 0:
         _check_packed(B, meta, s, prob_m, prob_k, lead=(batch,))
-    err = _ffi.lib().triteia_hip_bmm_2_4_tokens(
-        _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), prob_m, batch, tokens, prob_k,
-        _ffi.device_index(A), _ffi.stream_of(A))
+    if tokens == 1:
+        # the reference's own case and argument list (triteia_nm_bmm.cu:760-764)
+        if workspace.numel() < prob_m // 128 * max_par:
+            raise RuntimeError(f"workspace must be of size at least {prob_m // 128 * max_par}.")
+        err = _ffi.lib().triteia_hip_bmm_2_4(
+            _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), prob_m, batch, prob_k,
+            _ffi.ptr(workspace), groupsize, _ffi.device_index(A), _ffi.stream_of(A), thread_k, thread_m, sms, max_par)
+    else:
+        err = _ffi.lib().triteia_hip_bmm_2_4_tokens(
+            _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), prob_m, batch, tokens, prob_k,
+            _ffi.device_index(A), _ffi.stream_of(A))
     _raise(err, prob_m, batch, prob_k, thread_k, thread_m, groupsize)
 
 
@@ -105,10 +113,12 @@ def sbmm_2_4(A, B, meta, C, s, indices, workspace, starts, counts, thread_k=-1, 
     groupsize = -1 if s.shape[1] == 1 else prob_k // s.shape[1]
     if prob_m % 128 == 0 and prob_k % 64 == 0 and groupsize == -1:
         _check_packed(B, meta, s, prob_m, prob_k, lead=(B.shape[0],))
-    err = _ffi.lib().triteia_hip_sbmm_2_4(
+    # (the entry point with the reference's exact argument list, triteia_hip_sbmm_2_4, trusts the indices; this
+    # binding knows how many matrices B holds and passes it on, so that a stray index is skipped)
+    err = _ffi.lib().triteia_hip_sbmm_2_4_bounded(
         _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), _ffi.ptr(indices), _ffi.ptr(starts),
-        _ffi.ptr(counts), prob_m, prob_n, prob_k, indices.numel(), B.shape[0], _ffi.ptr(workspace), groupsize,
-        _ffi.device_index(A), _ffi.stream_of(A), thread_k, thread_n, sms, max_par)
+        _ffi.ptr(counts), prob_m, prob_n, prob_k, indices.numel(), _ffi.ptr(workspace), groupsize,
+        _ffi.device_index(A), _ffi.stream_of(A), thread_k, thread_n, sms, max_par, B.shape[0])
     _raise(err, prob_m, prob_n, prob_k, thread_k, thread_n, groupsize, knob="thread_n")
 
 
