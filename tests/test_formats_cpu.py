@@ -41,6 +41,30 @@ def test_gptq_dequantise_matches_a_plain_loop():
         unpack_4bit_to_32bit_signed(qweight, gptq_tensors(k, m, 1, zero=6)[2])
 
 
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_gptq_unpack_grouped_against_a_plain_loop(bits):
+    """scales[g] * (q - (zero + 1 mod 2^bits)) element by element, two groups along k, any zero point."""
+    k, m, per = 64, 32, 32 // bits
+    rng = np.random.default_rng(bits)
+    q = rng.integers(0, 1 << bits, size=(k, m))
+    zero = rng.integers(0, 1 << bits, size=(2, m))
+    scales = rng.uniform(0.005, 0.02, size=(2, m)).astype(np.float16)
+    qweight = np.zeros((k // per, m), dtype=np.uint64)
+    for row in range(k):
+        qweight[row // per] |= q[row].astype(np.uint64) << np.uint64(bits * (row % per))
+    qzeros = np.zeros((2, m // per), dtype=np.uint64)
+    for col in range(m):
+        qzeros[:, col // per] |= zero[:, col].astype(np.uint64) << np.uint64(bits * (col % per))
+    as_i32 = lambda a: torch.from_numpy(a.astype(np.uint32).view(np.int32))
+    got = gptq_unpack(bits, as_i32(qweight), as_i32(qzeros), torch.from_numpy(scales), group_size=k // 2)
+    want = np.empty((k, m), dtype=np.float16)
+    for row in range(k):
+        g = row // (k // 2)
+        for col in range(m):
+            want[row, col] = scales[g, col] * np.float16(int(q[row, col]) - ((int(zero[g, col]) + 1) % (1 << bits)))
+    assert got.shape == (k, m) and np.array_equal(got.numpy(), want)
+
+
 def llama_state_dict(hidden, inter, seed):
     sd, dense = {}, {}
     shapes = {"self_attn.q_proj": (hidden, hidden), "self_attn.k_proj": (hidden, hidden), "self_attn.v_proj": (hidden, hidden),

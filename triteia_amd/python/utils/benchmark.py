@@ -9,50 +9,56 @@ import torch
 from triteia_amd.python.configs.gpus import get_gpu_device_info
 
 
-def timing_function(func, flops_func, kwargs, repeats=1):
-    """Time `func(**kwargs restricted to its parameters)` with device events, `repeats` times.
+def _accepted(fn, kwargs):
+    """The entries of `kwargs` that `fn` names as parameters."""
+    names = inspect.signature(fn).parameters
+    return {name: value for name, value in kwargs.items() if name in names}
 
-    Units follow the reference: elapsed in ms, total_flops in GFLOP, perf_flops in GFLOP/s,
-    mfu in percent of the device's fp16 peak (None without a known device)."""
-    func_args_names = inspect.getfullargspec(func).args
-    func_args = {arg: kwargs[arg] for arg in func_args_names if arg in kwargs}
-    gpu_info = get_gpu_device_info()
-    flops_func_args = {}
-    if flops_func:
-        flops_func_args = {arg: kwargs[arg] for arg in inspect.getfullargspec(flops_func).args if arg in kwargs}
-    measurements = {"elapsed": [], "perf_flops": [], "mfu": []}
+
+def timing_function(func, flops_func, kwargs, repeats=1):
+    """Time `func` on the entries of `kwargs` it takes, `repeats` times, and report in the reference's
+    result schema (triteia/python/utils/benchmark.py:52-61: the keys below; elapsed in ms, total_flops in
+    GFLOP, perf_flops in GFLOP/s, mfu in percent of the device's fp16 peak or None for an unknown device).
+
+    All repeats are enqueued back to back, each between its own pair of events, and the events are read
+    once at the end: no host synchronisation falls between two timed calls."""
+    call_args = _accepted(func, kwargs)
+    flops = float(flops_func(**_accepted(flops_func, kwargs))) if flops_func else None
+    peak = (get_gpu_device_info() or {}).get("fp16_tflops")
+
+    marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(max(repeats, 1))]
     output = None
-    for _ in range(repeats):
-        torch.cuda.synchronize()
-        start = torch.cuda.Event(enable_timing=True)
-        end = torch.cuda.Event(enable_timing=True)
-        start.record()
-        output = func(**func_args)
+    torch.cuda.synchronize()
+    for begin, end in marks:
+        begin.record()
+        output = func(**call_args)
         end.record()
-        torch.cuda.synchronize()
-        elapsed = start.elapsed_time(end)
-        measurements["elapsed"].append(elapsed)
-        if flops_func:
-            total_flops = flops_func(**flops_func_args)
-            measurements["perf_flops"].append((total_flops / elapsed) / 1e6)
-            if gpu_info:
-                measurements["mfu"].append(100 * (total_flops / elapsed) / 1e9 / gpu_info["fp16_tflops"])
-    elapsed = sum(measurements["elapsed"]) / repeats
-    total_flops = perf_flops = mfu = None
-    if flops_func:
-        total_flops = flops_func(**flops_func_args)
-        perf_flops = total_flops / elapsed
-        if gpu_info:
-            mfu = 100 * perf_flops / 1e9 / gpu_info["fp16_tflops"]
+    torch.cuda.synchronize()
+    times_ms = [begin.elapsed_time(end) for begin, end in marks]
+
+    def rates(ms):
+        """(GFLOP/s, % of peak) of one duration."""
+        if flops is None:
+            return None, None
+        gflops = flops / ms / 1e6
+        return gflops, (100.0 * gflops / 1e3 / peak if peak else None)
+
+    per_call = [rates(ms) for ms in times_ms]
+    mean_ms = sum(times_ms) / len(times_ms)
+    mean_gflops, mean_mfu = rates(mean_ms)
     return {
         "output": output,
-        "elapsed": elapsed,
+        "elapsed": mean_ms,
         "func_name": func.__name__,
-        "total_flops": total_flops / 1e9 if flops_func else None,
-        "perf_flops": perf_flops / 1e6 if flops_func else None,
-        "mfu": mfu,
+        "total_flops": flops / 1e9 if flops is not None else None,
+        "perf_flops": mean_gflops,
+        "mfu": mean_mfu,
         "args": kwargs,
-        "measurements": measurements,
+        "measurements": {
+            "elapsed": times_ms,
+            "perf_flops": [g for g, _ in per_call if g is not None],
+            "mfu": [u for _, u in per_call if u is not None],
+        },
     }
 
 

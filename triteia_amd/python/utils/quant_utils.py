@@ -35,17 +35,17 @@ def dequantize_weight(qweight, qzeros, scales):
 
 @torch.no_grad()
 def gptq_unpack(bits, qweight, qzeros, scales, group_size=-1):
-    """General GPTQ unpack for 2/4/8 bits: scales * (q - (zero + 1)) as [k, m] (quant_utils.py:49-76)."""
+    """General GPTQ unpack for 2/4/8 bits: scales * (q - (zero + 1)) as [k, m] (quant_utils.py:49-76).
+
+    qweight int32 [k*bits/32, m] holds 32/bits values per word along k (lowest bits first), qzeros int32
+    [g, m*bits/32] the same along m, scales [g, m]; `zero + 1` wraps inside `bits` bits, as in the reference."""
+    per_word, mask = 32 // bits, (1 << bits) - 1
+    k, m = qweight.shape[0] * per_word, qweight.shape[1]
     if group_size == -1:
-        group_size = qweight.shape[0] * 32 // bits
-    wf = torch.arange(0, 32, bits, dtype=torch.int32, device=qweight.device).unsqueeze(0)
-    store = torch.int16 if bits == 8 else torch.int8
-    zeros = torch.bitwise_right_shift(qzeros.unsqueeze(2).expand(-1, -1, 32 // bits), wf.unsqueeze(0)).to(store)
-    zeros = torch.bitwise_and(zeros + 1, (2 ** bits) - 1)
-    zeros = zeros.reshape(-1, 1, zeros.shape[1] * zeros.shape[2])
-    scales = scales.reshape(-1, 1, scales.shape[-1])
-    weight = torch.bitwise_right_shift(qweight.unsqueeze(1).expand(-1, 32 // bits, -1), wf.unsqueeze(-1)).to(store)
-    weight = torch.bitwise_and(weight, (2 ** bits) - 1)
-    weight = weight.reshape(-1, group_size, weight.shape[2])
-    weight = scales * (weight - zeros)
-    return weight.reshape(weight.shape[0] * weight.shape[1], weight.shape[2])
+        group_size = k
+    shifts = torch.arange(per_word, dtype=torch.int32, device=qweight.device) * bits
+    q = ((qweight.unsqueeze(1) >> shifts.view(1, per_word, 1)) & mask).reshape(k, m)              # row per_word*i + j
+    z = ((qzeros.unsqueeze(2) >> shifts.to(qzeros.device).view(1, 1, per_word)) & mask).reshape(qzeros.shape[0], -1)
+    z = (z + 1) & mask
+    groups = scales.reshape(-1, scales.shape[-1])
+    return groups.repeat_interleave(group_size, dim=0) * (q - z.repeat_interleave(group_size, dim=0))
