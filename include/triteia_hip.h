@@ -126,7 +126,22 @@ TRITEIA_HIP_API int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, co
                                 void* stream);
 TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n_deltas);
 
-/* Only the routing step of the call above: fills `workspace` (16-byte aligned) with
+/* triteia_hip_sbmm_2_4_routed without the workspace argument, for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses that forbid it).  It
+ * has no counterpart in the reference.  The routing plan lives in a buffer inside the library's own
+ * device image (triteia_hip_sbmm_routed_static_max_bytes() = 256 KiB per GPU, held until the process
+ * ends); the call allocates and frees nothing.  Batches whose plan
+ * (triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas)) does not fit return
+ * TRITEIA_HIP_ERR_KERN_SHAPE: 8192 tokens over 1024 deltas fit, 65536 tokens over 64 deltas do not.
+ * Every call on one GPU uses that GPU's one buffer: calls that overlap in time on the same GPU
+ * (different streams, or one stream's call not finished when another's starts) race on it; calls in
+ * stream order on one stream are safe.  Results are those of triteia_hip_sbmm_2_4_routed, bit for bit. */
+TRITEIA_HIP_API int triteia_hip_sbmm_2_4_routed_static(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                       const void* token_indices, int index_offset, int n_deltas, int prob_m,
+                                       int prob_n, int prob_k, int accumulate, int dev, void* stream);
+TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_static_max_bytes(void);
+
+/* Only the routing step of triteia_hip_sbmm_2_4_routed: fills `workspace` (16-byte aligned) with
  *   int32 header[8] = {narrow tiles, routed tokens, deltas in use, narrow tile size,
  *                      wide tiles, tiles of all[], 0, 0}
  *   int32 tiles[max_tiles][4] = {delta, start, count, 0}: at most `tile size` tokens of one

@@ -312,6 +312,33 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   return TRITEIA_HIP_OK;
 }
 
+// Routing-plan scratch of triteia_hip_sbmm_2_4_routed_static: owned by the library, one copy per GPU (each
+// device that loads this code object holds its own instance of the array at its own address).  In host code
+// the array's name is only a handle for hipGetSymbolAddress; kernels get the per-device address it returns.
+constexpr size_t kStaticPlanBytes = 256 * 1024;
+__device__ __align__(256) unsigned char g_static_plan[kStaticPlanBytes];
+
+constexpr int kMaxDevices = 64;
+void* g_static_plan_addr[kMaxDevices] = {};
+std::mutex g_static_plan_mutex;
+
+// Address of the current device's instance of g_static_plan (looked up once per device, with that device current).
+int static_plan_address(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(TRITEIA_HIP_ERR_RUNTIME, "sbmm_2_4_routed_static: no current device");
+  std::lock_guard<std::mutex> lock(g_static_plan_mutex);
+  if (!g_static_plan_addr[dev]) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_plan));
+    if (e != hipSuccess || !ptr)
+      return fail(TRITEIA_HIP_ERR_RUNTIME, "sbmm_2_4_routed_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_static_plan_addr[dev] = ptr;
+  }
+  *out = g_static_plan_addr[dev];
+  return TRITEIA_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -586,6 +613,28 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   if (int e = triteia_hip_route_plan(token_indices, index_offset, n_deltas, prob_n, workspace, workspace_bytes, dev, stream))
     return e;
   return triteia_hip_sbmm_2_4_planned(A, B, meta, C, s, workspace, n_deltas, prob_m, prob_n, prob_k, accumulate, dev, stream);
+}
+
+size_t triteia_hip_sbmm_routed_static_max_bytes(void) { return kStaticPlanBytes; }
+
+int triteia_hip_sbmm_2_4_routed_static(const void* A, const void* B, const void* meta, void* C, const void* s,
+                                       const void* token_indices, int index_offset, int n_deltas, int prob_m,
+                                       int prob_n, int prob_k, int accumulate, int dev, void* stream) {
+  if (prob_n < 0 || n_deltas < 0)
+    return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sbmm_2_4_routed_static: tokens=%d deltas=%d", prob_n, n_deltas);
+  const size_t need = triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas);
+  if (need > kStaticPlanBytes)
+    return fail(TRITEIA_HIP_ERR_KERN_SHAPE,
+                "sbmm_2_4_routed_static: the routing plan of %d tokens over %d deltas takes %zu bytes, the library's "
+                "scratch holds %zu; use triteia_hip_sbmm_2_4_routed with a workspace of the caller's",
+                prob_n, n_deltas, need, kStaticPlanBytes);
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  void* plan = nullptr;
+  if (int e = static_plan_address(&plan)) return e;
+  // (the plan kernel writes every word of the plan that the multiply kernels read: nothing to clear)
+  return triteia_hip_sbmm_2_4_routed(A, B, meta, C, s, token_indices, index_offset, n_deltas, prob_m, prob_n, prob_k, plan,
+                                     kStaticPlanBytes, accumulate, -1, stream);
 }
 
 int triteia_hip_bgmv(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,

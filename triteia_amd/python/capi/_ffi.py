@@ -29,6 +29,8 @@ SIGNATURES = {
     "triteia_hip_sbmm_2_4": (_c_int, [_c_vp] * 8 + [_c_int] * 4 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
     "triteia_hip_sbmm_2_4_bounded": (_c_int, [_c_vp] * 8 + [_c_int] * 4 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 5),
     "triteia_hip_sbmm_2_4_routed": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_vp, _c_sz, _c_int, _c_int, _c_vp]),
+    "triteia_hip_sbmm_2_4_routed_static": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_int, _c_int, _c_vp]),
+    "triteia_hip_sbmm_routed_static_max_bytes": (_c_sz, []),
     "triteia_hip_sbmm_2_4_planned": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_int, _c_vp]),
     "triteia_hip_sbmm_routed_workspace_bytes": (_c_sz, [_c_int, _c_int]),
     "triteia_hip_plan_tile_tokens": (_c_int, [_c_int, _c_int]),
