@@ -13,6 +13,7 @@
 #include "lora.hip.h"
 #include "route_plan.hip.h"
 #include "sparse24_gemm.hip.h"
+#include "sparse24_tile256.hip.h"
 #include "sparse24_wide.hip.h"
 
 namespace {
@@ -20,6 +21,7 @@ namespace {
 using namespace triteia_hip;
 
 thread_local char g_err[512] = "";
+constexpr int kMaxDevicesForAttr = 64;
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -57,7 +59,7 @@ struct Knobs {
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
   int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
-  int tile256 = 1, tile256_min_units = kUnset, ksplit = 1;
+  int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1;
 };
 Knobs g_knobs;
 std::once_flag g_knobs_once;
@@ -72,7 +74,7 @@ void read_knobs() {
       {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
       {"MID_MIN_UNITS", &k.mid_min_units}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
-      {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units},
+      {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
       {"KSPLIT", &k.ksplit},
   };
   char name[64];
@@ -238,6 +240,38 @@ int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   return check_launch("sparse24_wide_kernel");
 }
 
+// 256-token x 256-column tiles on workgroups of eight wavefronts (153 KB of dynamic LDS, one workgroup per CU):
+// uniform groups only.
+bool g_tile256_ready[kMaxDevicesForAttr] = {};
+std::mutex g_tile256_mutex;
+int launch_tile256(const Sparse24Args& a, hipStream_t st) {
+  if (a.n_groups <= 0 || a.m == 0 || a.k == 0 || a.uniform_count <= 0) return TRITEIA_HIP_OK;
+  const long ncp = (a.m / 128 + 1) / 2;
+  const long tiles = (long)a.n_groups * ((a.uniform_count + kT256Tokens - 1) / kT256Tokens);
+  const long units = t256_grid(tiles, ncp);
+  if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
+  {
+    // more than 64 KB of LDS has to be granted once per device
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevicesForAttr)
+      return fail(TRITEIA_HIP_ERR_RUNTIME, "sparse24_tile256_kernel: no current device");
+    std::lock_guard<std::mutex> lock(g_tile256_mutex);
+    if (!g_tile256_ready[dev]) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse24_tile256_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kT256LdsBytes) != hipSuccess)
+        return fail(TRITEIA_HIP_ERR_RUNTIME, "sparse24_tile256_kernel: cannot reserve %d bytes of LDS", kT256LdsBytes);
+      g_tile256_ready[dev] = true;
+    }
+  }
+  hipLaunchKernelGGL(sparse24_tile256_kernel, dim3((unsigned)units), dim3(512), kT256LdsBytes, st, a);
+  return check_launch("sparse24_tile256_kernel");
+}
+// (token tile, column pair) units for which a uniform launch takes this kernel: launches of about one round of workgroups
+// (one per CU).  Measured against 64-token tiles: 4096 tokens on 4096 x 4096 (256 units) 89.1 against 95.8 us, on
+// 8192 x 8192 (512 units) 290 against 294 us; 4096 x 11008 (688 units) 228 against 227 us; 8192 x 28672 (1792 units)
+// 994 against 950 us; 2048 tokens on 4096 x 4096 (128 units: half the CUs idle) 72 against 55 us.
+constexpr long kTile256MinUnits = 192, kTile256MaxUnits = 512;
+
 // The wide kernel pays off when there are enough tiles to occupy the GPU; below that the narrow
 // kernel's smaller units win.  Knob `wide` = 0 disables it; `wide_min_units` moves the threshold.
 bool wide_enabled() { return knobs().wide != 0; }
@@ -255,6 +289,20 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
   bool ks64 = false;   // the whole launch goes to 64-token tiles on workgroups of eight wavefronts
   // (the wide kernels address activations with 32-bit byte offsets)
   const bool x_below_4g = ((long)(n_groups - 1) * stride + tokens) * a.x_stride * 2 < (1L << 32);
+  // Groups of hundreds of tokens: 256-token x 256-column tiles whose wavefronts share the dequantised weights.
+  if (knobs().tile256 && wide_enabled() && x_below_4g) {
+    const long ncp = (a.m / 128 + 1) / 2;
+    const long min_units = knob_or(knobs().tile256_min_units, kTile256MinUnits);
+    int t = tokens / kT256Tokens * kT256Tokens;
+    if (tokens - t >= kT256Tokens / 2 || min_units <= 1) t = tokens;     // a rest of half a tile and more is a tile
+    const long units = (long)n_groups * ((t + kT256Tokens - 1) / kT256Tokens) * ncp;
+    if (t > 0 && units >= min_units && units <= knob_or(knobs().tile256_max_units, kTile256MaxUnits)) {
+      a.uniform_first = 0;
+      a.uniform_count = t;
+      if (int e = launch_tile256(a, st)) return e;
+      done = t;
+    }
+  }
   // A launch of at most two 32-token workgroups per CU, but of more than the narrow kernel fills well, is bound by
   // the latency of each workgroup's chain of steps, not by the matrix cores: there the 32-token build of the wide
   // kernel with two steps of weights in flight per wavefront beats both the narrow kernel and 64-token tiles.
@@ -273,11 +321,11 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
     // are ahead while they make one workgroup per CU at most (4096 x 4096 with 1280 / 1536 tokens 49.7 -> 44.2,
     // 50.8 -> 46.0 us; 4096 x 11008 with 384 / 640 tokens 47.2 -> 43.0, 51.4 -> 46.0 us; 8192 x 8192 with 768 tokens 88.7 ->
     // 72.5 us; 8192 x 28672 with 192 tokens 89.4 -> 73.0 us)
-    ks64 = wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= kWideTokens &&
+    ks64 = done == 0 && wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= kWideTokens &&
            units32 > knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits) &&
            (long)n_groups * ((tokens + kWideTokens - 1) / kWideTokens) * ((cgs + 7) / 8 * 8) <=
                knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits);
-    if (!ks64 && wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= 32 &&
+    if (done == 0 && !ks64 && wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= 32 &&
         units32 >= knob_or(knobs().wide32_min_units, kWide32MinUnits) &&
         units32 <= knob_or(knobs().wide32_max_units, kWide32MaxUnits)) {
       a.uniform_first = 0;
