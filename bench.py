@@ -11,9 +11,12 @@ weights come from HBM, not from the 256 MB Infinity Cache.
 
 Prints ONE JSON line.  `value` is dense-equivalent TFLOP/s (2 * routed_tokens * k * m per
 step, the reference's convention, meta/benchmarks/bench_sbmm.py:17) over the timed region;
-`roofline` scores the dominant kernel against HBM bandwidth with its duration measured live by
-HIP events; `cpu_baseline` is the CPU oracle (dequantise, then torch matmul per delta) timed on
-the host cores on a bounded sample of the same workload.
+`roofline` scores the dominant kernel against HBM bandwidth (or the sparse-fp16 matrix-core peak,
+whichever bounds the workload) with its duration measured live by HIP events; `sweep` holds the
+same two measurements for the metric's grid (tokens x deltas at the 7B shapes: the reference's
+meta/benchmarks/bench_sbmm.py:117-140 and benchmarks/bench_ldmm.py:97-123 sweep the same axes);
+`cpu_baseline` is the reference's CPU-expressible path (dequantise with the package's torch codec,
+then torch matmul of the rows routed to each delta) timed on all host cores on a bounded sample.
 """
 import argparse
 import ctypes
@@ -44,6 +47,7 @@ def parse():
     p.add_argument("--copies", type=int, default=0, help="distinct weight copies to rotate over (0 = auto)")
     p.add_argument("--no-graph", action="store_true", help="time eager launches instead of one captured HIP graph")
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-sweep", action="store_true", help="skip the tokens x deltas sweep (the `sweep` array)")
     p.add_argument("--warm-cache", action="store_true", help="do not rotate weight copies (Infinity-Cache-warm number)")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run one plain 256 MiB device copy (a known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -68,6 +72,11 @@ class Problem:
         self.ws = torch.zeros((nbytes + 3) // 4, dtype=torch.int32, device=dev)
         self.ws_bytes = self.ws.numel() * 4
         self.lock_ws = torch.zeros(max(wl.m, 16) * max(1, wl.n_deltas), dtype=torch.int32, device=dev)
+        # matmul / bmm launches of few workgroups split K across workgroups through a scratch buffer of the caller's
+        groups, per_group = (1, wl.tokens) if wl.op == "matmul" else (wl.n_deltas, max(1, wl.tokens // max(1, wl.n_deltas)))
+        nb = self.lib.triteia_hip_bmm_scratch_bytes(wl.m, groups, per_group, wl.k) if wl.op in ("matmul", "bmm") else 0
+        self.scratch = torch.empty(max(nb, 16), dtype=torch.uint8, device=dev)
+        self.scratch_bytes = nb
         if wl.op == "ldmm":
             g = torch.Generator(device=dev).manual_seed(wl.seed + 3)
             self.base = [(torch.randn((wl.m, wl.k), generator=g, device=dev) * 0.02).half() for _ in range(copies)]
@@ -102,9 +111,15 @@ class Problem:
         wl, P = self.wl, self.ffi.ptr
         q, me, s = self.weights[i % self.copies]
         st = self.stream()
-        if wl.op == "matmul":
+        if wl.op == "matmul" and self.scratch_bytes:
+            self._chk(self.lib.triteia_hip_bmm_2_4_tokens_scratch(P(self.x), P(q), P(me), P(self.out), P(s), wl.m, 1, wl.tokens, wl.k,
+                                                                  P(self.scratch), self.scratch_bytes, 0, st))
+        elif wl.op == "matmul":
             self._chk(self.lib.triteia_hip_mul_2_4(P(self.x), P(q), P(me), P(self.out), P(s), wl.m, wl.tokens, wl.k, P(self.lock_ws),
                                                     -1, 0, st, -1, -1, -1, 16))
+        elif wl.op == "bmm" and self.scratch_bytes:
+            self._chk(self.lib.triteia_hip_bmm_2_4_tokens_scratch(P(self.x), P(q), P(me), P(self.out), P(s), wl.m, wl.n_deltas, 1, wl.k,
+                                                                  P(self.scratch), self.scratch_bytes, 0, st))
         elif wl.op == "bmm":
             self._chk(self.lib.triteia_hip_bmm_2_4(P(self.x), P(q), P(me), P(self.out), P(s), wl.m, wl.n_deltas, wl.k, P(self.lock_ws),
                                                     -1, 0, st, -1, -1, -1, 16))
@@ -175,43 +190,210 @@ class Problem:
 
 
 def cpu_baseline(wl, torch, budget_s=20.0):
-    """The CPU oracle on the host cores: numpy dequantise of packed deltas + torch matmul per
-    delta, on as many of the workload's deltas as fit the time budget, scaled to all of them."""
-    from oracle import triteia_oracle as orc
+    """The reference's CPU-expressible path on the host cores (its tests' own recipe: dequantise to a dense fp16
+    matrix, generator.py:40,52, then matmul per delta, sbmm.py:7-23): the package's vectorised torch codec
+    `unpack_2_4` and torch.matmul of the rows actually routed to each delta, on every host core, on as many of the
+    workload's deltas as fit the time budget (the rate is per delta and carries over to all of them)."""
     from triteia_amd import workloads as W
-    cores = min(os.cpu_count() or 1, 16)
+    from triteia_amd.python.ops.utils.sparsity import unpack_2_4
+    cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     didx = wl.delta_indices()
     used = sorted(set(int(i) for i in didx if i >= 0)) if didx is not None else list(range(wl.n_deltas))
-    counts = {d: (int((didx == d).sum()) if didx is not None else wl.tokens // wl.n_deltas) for d in used}
-    x = W.random_activations(wl.tokens, wl.k, wl.seed + 1, "cpu").float()
+    per_group = max(1, wl.tokens // max(1, wl.n_deltas))
+    x = W.random_activations(wl.tokens, wl.k, wl.seed + 1, "cpu")
     t_deq = t_mm = 0.0
     flops = 0.0
     done = 0
     t_begin = time.perf_counter()
     for d in used:
         q, me, s = W.random_packed_deltas(1, wl.k, wl.m, wl.seed + 31 * d, "cpu")
+        if didx is not None:
+            rows = x[torch.from_numpy(np.nonzero(didx == d)[0])]
+        elif wl.op == "bmm":
+            rows = x[d * per_group:(d + 1) * per_group]
+        else:
+            rows = x
         t0 = time.perf_counter()
-        dense = orc.unpack(q[0].numpy(), me[0].numpy(), s[0].numpy())
+        dense = unpack_2_4(q[0], me[0], s[0], dtype=torch.float32)
         t1 = time.perf_counter()
-        wt = torch.from_numpy(dense).float()
-        rows = x[: counts[d]]
-        y = rows @ wt
+        y = rows.float() @ dense
         t2 = time.perf_counter()
-        del y
+        del y, dense
         t_deq += t1 - t0
         t_mm += t2 - t1
-        flops += 2.0 * counts[d] * wl.k * wl.m
+        flops += 2.0 * rows.shape[0] * wl.k * wl.m
         done += 1
         if time.perf_counter() - t_begin > budget_s:
             break
     total = t_deq + t_mm
     return {
         "value": round(flops / total / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-        "sample": f"{done} of {len(used)} routed deltas of the workload (numpy dequantise {t_deq:.2f}s on 1 thread + torch fp32 "
-                  f"matmul {t_mm:.3f}s on {cores} threads); the rate is per delta and carries over to all of them",
+        "sample": f"{done} of {len(used)} routed deltas of the workload: torch dequantise {t_deq:.2f}s + torch fp32 matmul of the "
+                  f"rows routed to each delta {t_mm:.3f}s, both on {cores} threads; the rate is per delta and carries over to all of them",
         "dequant_s": round(t_deq, 3), "matmul_s": round(t_mm, 4),
     }
+
+
+def kernel_name(wl, lib, in_kernel):
+    """The kernel that takes most of the workload's rows, as the library itself reports it."""
+    if wl.op in ("matmul", "bmm"):
+        groups, per_group = (1, wl.tokens) if wl.op == "matmul" else (wl.n_deltas, max(1, wl.tokens // max(1, wl.n_deltas)))
+        code = lib.triteia_hip_uniform_kernel(wl.m, groups, per_group, wl.k, 1)
+        if code >= 1000:
+            return f"sparse24_grouped_kernel (K split over {code - 1000} workgroups) + splitk_reduce_kernel"
+        return {0: "sparse24_grouped_kernel", 32: "sparse24_wide_kernel<32 tokens>", 33: "sparse24_wide_kernel<32 tokens, 8 wavefronts>",
+                64: "sparse24_wide_kernel<64 tokens>", 65: "sparse24_wide_kernel<64 tokens, 8 wavefronts>",
+                256: "sparse24_tile256_kernel"}.get(code, f"kernel code {code}")
+    if in_kernel:
+        return "sparse24_grouped_kernel (routes in-kernel)"
+    if wl.index_offset:
+        return "sparse24_grouped_kernel"
+    tk = lib.triteia_hip_planned_tile_kernel(wl.tokens, wl.n_deltas, wl.m, wl.k)
+    if tk:
+        return f"sparse24_wide_kernel<{tk}-token plan tiles>"
+    hot = wl.tokens >= 256 and wl.tokens >= 8 * min(wl.tokens, wl.n_deltas)
+    return "sparse24_grouped_kernel" + (" + sparse24_wide_kernel<64-token tiles of hot deltas>" if hot else "")
+
+
+def measure(prob, wl, torch, ffi, steps, warmup, use_graph=True, reps=None):
+    """One workload: the step timed over `steps` steps (one captured HIP graph, or eager), and its dominant kernel
+    timed on its own by HIP events on the launch stream."""
+    lib = ffi.lib()
+    for i in range(warmup):
+        prob.step(i)
+    torch.cuda.synchronize()
+    if use_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(steps):
+                    prob.step(warmup + i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        del graph
+    else:
+        t0 = time.perf_counter()
+        for i in range(steps):
+            prob.step(warmup + i)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    step_s = elapsed / steps
+
+    # ---- dominant kernel alone: batches of back-to-back launches between two events
+    # (a batch that the routed entry point routes inside the multiply kernel is one launch: the whole step; otherwise
+    # the multiply runs on a routing plan made beforehand)
+    in_kernel = wl.op == "sbmm" and bool(lib.triteia_hip_routed_in_kernel(wl.tokens, wl.n_deltas, wl.m, wl.k))
+    kernel_call = prob.step if in_kernel else (prob.delta_routed if wl.index_offset else prob.delta_kernel)
+    if wl.indices is not None and not in_kernel:
+        prob.plan()
+    for i in range(5):
+        kernel_call(i)
+    torch.cuda.synchronize()
+    batch = 10
+    reps = reps or max(3, min(20, steps // 10))
+    durs = []
+    for r in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(batch):
+            kernel_call(r * batch + i)
+        e1.record()
+        e1.synchronize()
+        durs.append(e0.elapsed_time(e1) / batch * 1e-3)
+    kdur = float(np.median(durs))
+    abytes = wl.delta_algorithmic_bytes()
+    achieved = abytes / kdur / 1e9
+    kflops = wl.delta_flops() / kdur / 1e12
+    name = kernel_name(wl, lib, in_kernel)
+    hbm_time, mfma_time = abytes / (HBM_PEAK_GBS * 1e9), wl.delta_flops() / (MFMA_SPARSE_F16_TFLOPS * 1e12)
+    if mfma_time > hbm_time:
+        # many tokens per delta: the matrix cores bound the kernel.  The 2:4-sparse instruction executes
+        # half of the dense-equivalent multiply-adds, priced against the dense fp16 peak (same fraction
+        # as dense-equivalent work against twice that peak).
+        roofline = {
+            "bound": "mfma", "achieved": round(kflops / 2, 1), "peak": MFMA_SPARSE_F16_TFLOPS / 2, "unit": "TFLOP/s",
+            "frac": round(kflops / MFMA_SPARSE_F16_TFLOPS, 4), "traffic": None, "kernel": name, "kernel_us": round(kdur * 1e6, 2),
+            "algorithmic_flops_dense_equivalent": wl.delta_flops(), "kernel_tflops_dense_equivalent": round(kflops, 2),
+            "hbm_frac": round(achieved / HBM_PEAK_GBS, 4),
+        }
+    else:
+        roofline = {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None, "kernel": name, "kernel_us": round(kdur * 1e6, 2), "algorithmic_bytes": abytes,
+            "kernel_tflops": round(kflops, 2), "mfma_frac": round(kflops / MFMA_SPARSE_F16_TFLOPS, 4),
+        }
+    return step_s, roofline
+
+
+def copies_for(wl, warm=False, asked=0):
+    """Distinct weight copies to rotate over: enough bytes to out-run the 256 MB Infinity Cache, within ~12 GB."""
+    if warm:
+        return 1
+    if asked > 0:
+        return asked
+    touched = wl.distinct_deltas() * wl.delta_bytes
+    return max(1, min(64, int(np.ceil(1.5 * 2 ** 30 / max(touched, 1))), int(12 * 2 ** 30 // (wl.n_deltas * wl.delta_bytes)) or 1))
+
+
+def sweep_points():
+    """The metric's grid: routed sbmm over 16 deltas of 4096 x 4096 and over 32 deltas of 4096 x 11008 against the token
+    count, the single-matrix product at three token counts, and the ldmm step of configuration 3."""
+    from triteia_amd import workloads as W
+    pts = []
+    for t in (1, 16, 64, 256, 1024, 4096):
+        pts.append((f"sbmm 16 x 4096x4096, {t} tokens", W.config("cfg2", t)))
+    for t in (1, 16, 64, 256, 1024, 4096):
+        wl = W.config("cfg3", t)
+        wl.op, wl.name = "sbmm", f"sbmm 32 x 4096x11008, {t} tokens Zipf(1.5) 10% -1"
+        pts.append((f"sbmm 32 x 4096x11008, {t} tokens", wl))
+    for t in (16, 1024, 4096):
+        pts.append((f"matmul 4096x4096, {t} tokens", W.config("cfg0", t)))
+    pts.append(("bmm 8 x 4096x4096, 1 token each (cfg1)", W.config("cfg1")))
+    pts.append(("ldmm 4096x11008, 256 tokens (cfg3)", W.config("cfg3")))
+    return pts
+
+
+def run_sweep(torch, ffi):
+    out = []
+    for label, wl in sweep_points():
+        prob = Problem(wl, copies_for(wl), torch, ffi)
+        torch.cuda.synchronize()
+        # a few milliseconds of steps per point
+        est_us = max(10.0, wl.delta_flops() / 1.5e15 * 1e6, wl.delta_algorithmic_bytes() / 4e12 * 1e6)
+        steps = int(min(50, max(10, 4000.0 / est_us)))
+        step_s, roof = measure(prob, wl, torch, ffi, steps, 3, use_graph=True, reps=5)
+        flops = wl.delta_flops()
+        if wl.op == "ldmm":
+            flops += 2.0 * wl.tokens * wl.k * wl.m + 2.0 * wl.lora_tokens() * wl.lora_rank * (wl.k + wl.m)
+        out.append({"workload": label, "tokens": wl.tokens, "tokens_routed": wl.routed_tokens(), "deltas_used": wl.distinct_deltas(),
+                    "ms_per_step": round(step_s * 1e3, 5), "tflops": round(flops / step_s / 1e12, 2), "kernel": roof["kernel"],
+                    "kernel_us": roof["kernel_us"], "bound": roof["bound"], "frac": roof["frac"]})
+        del prob
+        torch.cuda.empty_cache()
+    return out
+
+
+def host_call_us(prob, wl, torch, n=300):
+    """Host time of one `ops.sbmm_4bit_2_4_native` call (Python mirror -> ctypes -> C ABI), launches left to queue up."""
+    if wl.op != "sbmm":
+        return None
+    from triteia_amd.python import ops
+    q, me, s = prob.weights[0]
+    for _ in range(20):
+        ops.sbmm_4bit_2_4_native(q, prob.x, me, s, prob.idx)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        ops.sbmm_4bit_2_4_native(q, prob.x, me, s, prob.idx)
+    host = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    return round(host / n * 1e6, 2)
 
 
 def main():
@@ -236,14 +418,7 @@ def main():
     if a.deltas is not None and a.workload == "cfg4":
         wl.n_deltas = a.deltas
         wl.indices = W.zipf_indices(wl.tokens, wl.n_deltas, 1.2, wl.seed)
-    touched = wl.distinct_deltas() * wl.delta_bytes
-    if a.warm_cache:
-        copies = 1
-    elif a.copies > 0:
-        copies = a.copies
-    else:
-        # enough distinct bytes to out-run the 256 MB Infinity Cache, within ~12 GB
-        copies = max(1, min(64, int(np.ceil(1.5 * 2 ** 30 / max(touched, 1))), int(12 * 2 ** 30 // (wl.n_deltas * wl.delta_bytes)) or 1))
+    copies = copies_for(wl, a.warm_cache, a.copies)
     prob = Problem(wl, copies, torch, ffi)
     torch.cuda.synchronize()
     if a.calibrate_copy:
@@ -254,30 +429,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # ---- whole-job timing: W warm-up steps, then exactly K steps
-    for i in range(a.warmup):
-        prob.step(i)
-    torch.cuda.synchronize()
+    # ---- whole-job timing (W warm-up steps, then exactly K steps) and the dominant kernel on its own
     use_graph = not a.no_graph
-    if use_graph:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            with torch.cuda.graph(graph, stream=side):
-                for i in range(a.steps):
-                    prob.step(a.warmup + i)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        graph.replay()
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-    else:
-        t0 = time.perf_counter()
-        for i in range(a.steps):
-            prob.step(a.warmup + i)
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
+    step_s, roofline = measure(prob, wl, torch, ffi, a.steps, a.warmup, use_graph)
     # eager launches too (shows the host launch cost next to the graph number)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -286,69 +440,23 @@ def main():
     torch.cuda.synchronize()
     eager = time.perf_counter() - t0
 
-    ms_per_step = elapsed / a.steps * 1e3
+    ms_per_step = step_s * 1e3
     flops = wl.delta_flops()
     if wl.op == "ldmm":
         flops += 2.0 * wl.tokens * wl.k * wl.m + 2.0 * wl.lora_tokens() * wl.lora_rank * (wl.k + wl.m)
-    value = flops / (elapsed / a.steps) / 1e12
-
-    # ---- dominant kernel alone: HIP events on the launch stream, batches of back-to-back launches
-    # (a batch of at most 64 tokens over at most 64 deltas, or of at most 256 tokens over at most 32 deltas,
-    # is routed inside the multiply kernel: the whole step is that one launch, and it is the kernel timed
-    # here; otherwise the multiply runs on a routing plan)
-    fused = wl.op == "sbmm" and ((wl.tokens <= 64 and wl.n_deltas <= 64) or (wl.tokens <= 256 and wl.n_deltas <= 32))
-    kernel_call = prob.step if fused else (prob.delta_routed if wl.index_offset else prob.delta_kernel)
-    if wl.indices is not None and not fused:
-        prob.plan()
-    for i in range(5):
-        kernel_call(i)
-    torch.cuda.synchronize()
-    batch, reps = 10, max(3, min(20, a.steps // 10))
-    durs = []
-    for r in range(reps):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(batch):
-            kernel_call(r * batch + i)
-        e1.record()
-        e1.synchronize()
-        durs.append(e0.elapsed_time(e1) / batch * 1e-3)
-    kdur = float(np.median(durs))
+    value = flops / step_s / 1e12
     abytes = wl.delta_algorithmic_bytes()
-    achieved = abytes / kdur / 1e9
-    kflops = wl.delta_flops() / kdur / 1e12
-    traffic = None
+
+    # HBM bytes per launch of the dominant kernel, from the committed rocprofv3 --pmc summary of this workload (two
+    # counter runs scaled by a plain copy of known size); the file names the commit it was measured at
     tpath = os.path.join(ROOT, "profiles", f"traffic_{a.workload}.json")
     if os.path.exists(tpath) and a.tokens is None and a.deltas is None and a.shape is None:
         try:
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+            tj = json.load(open(tpath))
+            roofline["traffic"] = tj.get("hbm_bytes_per_launch")
+            roofline["traffic_measured_at"] = tj.get("commit")
         except Exception:
-            traffic = None
-    # which kernel took the tiles (a plan's tiles on a wide layer run on a build of the wide kernel)
-    kernel_name = "sparse24_grouped_kernel"
-    if wl.indices is not None and not fused and not wl.index_offset:
-        tk = ffi.lib().triteia_hip_planned_tile_kernel(wl.tokens, wl.n_deltas, wl.m, wl.k)
-        if tk:
-            kernel_name = f"sparse24_wide_kernel<1, {tk}, true>"
-    hbm_time, mfma_time = abytes / (HBM_PEAK_GBS * 1e9), wl.delta_flops() / (MFMA_SPARSE_F16_TFLOPS * 1e12)
-    if mfma_time > hbm_time:
-        # many tokens per delta: the matrix cores bound the kernel.  The 2:4-sparse instruction executes
-        # half of the dense-equivalent multiply-adds, priced against the dense fp16 peak (same fraction
-        # as dense-equivalent work against twice that peak).
-        executed = kflops / 2
-        roofline = {
-            "bound": "mfma", "achieved": round(executed, 1), "peak": MFMA_SPARSE_F16_TFLOPS / 2, "unit": "TFLOP/s",
-            "frac": round(kflops / MFMA_SPARSE_F16_TFLOPS, 4), "traffic": traffic,
-            "kernel": "sparse24_wide128_kernel / sparse24_wide_kernel", "kernel_us": round(kdur * 1e6, 2),
-            "algorithmic_flops_dense_equivalent": wl.delta_flops(), "kernel_tflops_dense_equivalent": round(kflops, 2),
-            "hbm_frac": round(achieved / HBM_PEAK_GBS, 4),
-        }
-    else:
-        roofline = {
-            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": traffic, "kernel": kernel_name, "kernel_us": round(kdur * 1e6, 2), "algorithmic_bytes": abytes,
-            "kernel_tflops": round(kflops, 2), "mfma_frac": round(kflops / MFMA_SPARSE_F16_TFLOPS, 4),
-        }
+            pass
 
     # what this GPU delivers on a plain device-to-device copy (512 MiB read + 512 MiB written per launch), next to
     # the nominal peak the fractions above are priced against
@@ -375,9 +483,14 @@ def main():
                    "tokens": wl.tokens, "tokens_routed": wl.routed_tokens(), "weight_copies_rotated": copies,
                    "launch": "hip-graph" if use_graph else "eager"},
         "eager_ms_per_step": round(eager / a.steps * 1e3, 5),
-        "step_gbs": round((abytes + (wl.k * wl.m * 2 if wl.op == "ldmm" else 0)) / (elapsed / a.steps) / 1e9, 1),
+        "host_us_per_ops_call": host_call_us(prob, wl, torch),
+        "step_gbs": round((abytes + (wl.k * wl.m * 2 if wl.op == "ldmm" else 0)) / step_s / 1e9, 1),
         "roofline": roofline,
     }
+    del prob
+    torch.cuda.empty_cache()
+    if not a.no_sweep and a.workload == "cfg2" and a.tokens is None:
+        res["sweep"] = run_sweep(torch, ffi)
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl, torch)
     print(json.dumps(res))

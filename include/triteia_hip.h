@@ -83,6 +83,27 @@ TRITEIA_HIP_API int triteia_hip_bmm_2_4(const void* A, const void* B, const void
 TRITEIA_HIP_API int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
                                int batch, int tokens, int prob_k, int dev, void* stream);
 
+/* The same with a scratch buffer of the caller's (device memory, 16-byte aligned, contents irrelevant, overwritten),
+ * which lets a launch of few workgroups split K across workgroups: every workgroup writes the fp32 sums of its
+ * share of K to the buffer and a second, small launch adds the shares in a fixed order (the result is a function of
+ * the inputs only, but may differ in the last bit from the call without scratch, which adds over K in one
+ * workgroup).  triteia_hip_bmm_scratch_bytes says how many bytes the split of a launch uses (0: this launch would not
+ * be split and ignores the buffer); a smaller or null buffer simply leaves K unsplit.  batch = 1 is the single-matrix
+ * product.  The counterpart in the reference is the stripe partitioning of one GEMM over all SMs with its
+ * reduction through C under locks (triteia/csrc/ops/marlin.cuh:449-519, marlin_nm.cu:19-37): the lock array of its
+ * argument list is too small for fp32 partial sums, hence the separate argument here. */
+TRITEIA_HIP_API int triteia_hip_bmm_2_4_tokens_scratch(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
+                                       int batch, int tokens, int prob_k, void* scratch, size_t scratch_bytes, int dev,
+                                       void* stream);
+TRITEIA_HIP_API size_t triteia_hip_bmm_scratch_bytes(int prob_m, int batch, int tokens, int prob_k);
+
+/* Which kernel the uniform-group entry points (mul_2_4: batch = 1; bmm_2_4*) run most of a launch's rows on: 0 = the
+ * K-split streaming kernel (sparse24_grouped_kernel), 1000 + n = the same with K split over n workgroups (only
+ * with_scratch != 0), 32 / 64 = 32- / 64-token tiles of sparse24_wide_kernel (+ 1: on eight wavefronts), 256 =
+ * sparse24_tile256_kernel; -1 for a shape the entry points reject.  No counterpart in the reference; for benchmarks,
+ * profiles and the test that guards the dispatch thresholds. */
+TRITEIA_HIP_API int triteia_hip_uniform_kernel(int prob_m, int batch, int tokens, int prob_k, int with_scratch);
+
 /* Run-list form: for run r < prob_r, rows starts[r] .. starts[r]+counts[r]-1 of
  * C = same rows of A @ dequant(B[indices[r]]).  indices / starts / counts are
  * int32 device arrays.  Replaces triteia_cuda_sbmm_2_4
@@ -170,6 +191,11 @@ TRITEIA_HIP_API int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas);
  * the reference; for benchmarks and profiles, and for tests that compare results bit for bit (the two
  * kernels add over K in different orders). */
 TRITEIA_HIP_API int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k);
+
+/* 1 if triteia_hip_sbmm_2_4_routed handles this batch and layer in one launch, routing inside the multiply kernel
+ * (the workspace stays untouched), 0 if it builds a routing plan first.  No counterpart in the reference; for
+ * benchmarks and profiles. */
+TRITEIA_HIP_API int triteia_hip_routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k);
 
 /* The multiply step alone, on a plan made by triteia_hip_route_plan for the same
  * (prob_n, n_deltas): C[t] (+)= A[t] @ dequant(B[d]) for every routed token.  One

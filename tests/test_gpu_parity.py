@@ -110,6 +110,77 @@ def test_matmul_many_tokens_reference_test_shape(ops):
     check_close(out, ref, what="matmul 4096^3")
 
 
+@pytest.mark.parametrize("b,n,k,m,ks,seed", [
+    (1, 16, 8192, 256, 0, 40),                          # a long K on a narrow layer: split by the default rule
+    (1, 1, 512, 256, 2, 41), (1, 16, 512, 384, 3, 42),  # forced splits; 3 does not divide the 4 steps
+    (1, 40, 1024, 256, 4, 43), (1, 100, 448, 128, 2, 44),  # several token passes; a partial last step of K
+    (1, 8, 192, 256, 5, 45),                            # more splits asked for than there are steps
+    (3, 5, 512, 256, 2, 46), (4, 1, 8192, 128, 0, 47),  # bmm, forced and by the rule
+])
+def test_split_k_across_workgroups(ops, monkeypatch, b, n, k, m, ks, seed):
+    """matmul / bmm launches of few workgroups split K across workgroups (fp32 partial sums in a scratch buffer, added
+    in a fixed order by a second launch): against the oracle, against the unsplit kernel, and the same bits on every
+    one of 20 calls."""
+    say(f"split-K b={b} n={n} k={k} m={m} forced={ks} seed={seed}")
+    from triteia_amd.python.capi import _ffi
+    if ks:
+        setknob(monkeypatch, "TRITEIA_HIP_KSPLIT", ks)
+    kind = _ffi.lib().triteia_hip_uniform_kernel(m, b, n, k, 1)
+    assert kind > 1000, f"this launch is meant to be split (kernel code {kind})"
+    qw, meta, s = make_deltas(b, k, m, seed)
+    x = activations(b * n, k, seed + 1).reshape(b, n, k)
+    gq, gm, gs, gx = to_gpu(qw, meta, s, x)
+    if b == 1:
+        ref = orc.matmul_4bit_2_4(qw[0], x[0], meta[0], s[0])
+        call = lambda: ops.matmul_4bit_2_4(gq[0], gx[0], gm[0], gs[0])
+    else:
+        ref = orc.bmm_4bit_2_4(qw, x, meta, s)
+        call = lambda: ops.bmm_4bit_2_4(gq, gx, gm, gs)
+    first = call()
+    torch.cuda.synchronize()
+    check_close(first, ref, what="split-K")
+    for _ in range(19):
+        again = call()
+        assert torch.equal(again, first), "the K split must not depend on the order in which workgroups finish"
+    setknob(monkeypatch, "TRITEIA_HIP_KSPLIT", 0)          # 0 turns the split off
+    assert _ffi.lib().triteia_hip_uniform_kernel(m, b, n, k, 1) < 1000
+    unsplit = call()
+    torch.cuda.synchronize()
+    assert float((first.float() - unsplit.float()).norm() / unsplit.float().norm()) < 1e-4
+
+
+def test_reference_shaped_entry_points_directly(ops):
+    """triteia_hip_mul_2_4, triteia_hip_bmm_2_4 and triteia_hip_sbmm_2_4 called with exactly the reference launchers'
+    argument lists (marlin_nm.cu:42-46, triteia_nm_bmm.cu:760-764, triteia_nm_sbmm.cu:809-815), no binding layer."""
+    say("reference-shaped C entry points")
+    from triteia_amd.python.capi import _ffi
+    lib, P = _ffi.lib(), _ffi.ptr
+    b, k, m = 6, 512, 384
+    qw, meta, s = make_deltas(b, k, m, 61)
+    x = activations(b, k, 62)
+    gq, gm, gs, gx = to_gpu(qw, meta, s, x)
+    ws = torch.zeros(m // 128 * 16 * b, dtype=torch.int32, device=DEV)
+    st = _ffi.stream_of(gx)
+    # mul_2_4: all rows through matrix 2
+    out = torch.zeros(b, m, dtype=torch.float16, device=DEV)
+    assert lib.triteia_hip_mul_2_4(P(gx), P(gq[2]), P(gm[2]), P(out), P(gs[2]), m, b, k, P(ws), -1, 0, st, -1, -1, -1, 16) == 0
+    check_close(out, orc.matmul_4bit_2_4(qw[2], x, meta[2], s[2]), what="triteia_hip_mul_2_4")
+    # bmm_2_4: row i through matrix i
+    out = torch.zeros(b, 1, m, dtype=torch.float16, device=DEV)
+    assert lib.triteia_hip_bmm_2_4(P(gx), P(gq), P(gm), P(out), P(gs), m, b, k, P(ws), -1, 0, st, -1, -1, -1, 16) == 0
+    check_close(out, orc.bmm_4bit_2_4(qw, x.reshape(b, 1, k), meta, s), what="triteia_hip_bmm_2_4")
+    # sbmm_2_4: runs {matrix 4: rows 0-1}, {matrix 1: rows 2-4}, {-1: row 5}
+    idx = np.array([4, 4, 1, 1, 1, -1], dtype=np.int32)
+    run_idx, run_start, run_count = to_gpu(np.array([4, 1, -1], dtype=np.int32), np.array([0, 2, 5], dtype=np.int32),
+                                           np.array([2, 3, 1], dtype=np.int32))
+    out = torch.zeros(b, m, dtype=torch.float16, device=DEV)
+    assert lib.triteia_hip_sbmm_2_4(P(gx), P(gq), P(gm), P(out), P(gs), P(run_idx), P(run_start), P(run_count), m, b, k, 3,
+                                    P(ws), -1, 0, st, -1, -1, -1, 16) == 0
+    torch.cuda.synchronize()
+    check_close(out, orc.sbmm_4bit_2_4(qw, x, meta, s, idx), what="triteia_hip_sbmm_2_4")
+    assert bool((out[5] == 0).all()) and int(ws.abs().sum()) == 0
+
+
 def test_matmul_leading_dims_and_module(ops):
     from triteia_amd.python.nn.linear import sparse_low_precision_linear
     say("matmul leading dims + nn module")

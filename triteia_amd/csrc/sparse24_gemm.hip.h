@@ -99,6 +99,12 @@ struct Sparse24Args {
   int raw_static;           // fused routing with group g = delta g: weights are requested before the indices arrive
   int rot_spread;           // steps between the starting points of consecutive deltas' walks over K (0: all start at step 0)
   int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run
+  // K split across workgroups (uniform groups only): blockIdx.z = z takes the steps [z * ksplit_steps, (z + 1) * ksplit_steps)
+  // of K and writes its fp32 sums, unscaled, to partial[z][row][column]; splitk_reduce_kernel adds the splits in
+  // the order of z and finishes the rows.  ksplit_steps = 0: no split.
+  float* partial;
+  long partial_rows;        // rows of one split's block in `partial` (= rows of `out`)
+  int ksplit_steps;
 };
 
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
@@ -170,6 +176,7 @@ struct TileCtx {
   long qrow, mrow;          // vectors per packed row (weights, metadata)
   int k_rows, n_steps;      // packed rows, 128-k steps
   int rot;                  // this delta's walk over K starts at step `rot` and wraps around
+  int step0;                // first step of this workgroup's share of K (K split across workgroups), else 0
   int cb;                   // column block
   int tid, wave, lane, r, q;
   // fused routing (up to kRawParts x 64 tokens, kRawParts per lane): for part j of the batch (tokens
@@ -194,7 +201,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   // stream at 4.8 TB/s in lockstep, at 5.7 TB/s with their walks spread around the ring).
   auto phys = [&](int st) {
     const int ps = st + c.rot;
-    return st < n_steps ? (ps < n_steps ? ps : ps - n_steps) : 0;
+    return c.step0 + (st < n_steps ? (ps < n_steps ? ps : ps - n_steps) : 0);
   };
 
   // Steps past the end of K (st >= n_steps) read step 0 again: cheap cache hits that keep the
@@ -373,6 +380,13 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 #pragma unroll
         for (int i = 0; i < 4; i++) { v[i] += a0[i]; v[4 + i] += a1[i]; }
       }
+      if (p.ksplit_steps) {
+        // this workgroup's share of K only: the sums go to its block of the partial buffer as they are
+        float* pp = p.partial + ((long)blockIdx.z * p.partial_rows + row) * p.m + c.cb * 128 + f0;
+        *reinterpret_cast<float4_t*>(pp) = float4_t{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<float4_t*>(pp + 4) = float4_t{v[4], v[5], v[6], v[7]};
+        continue;
+      }
       // (sv: f0 is the same for every chunk of a thread, 64 * KW being a multiple of 16)
       _Float16* op = p.out + (long)row * p.out_stride + c.cb * 128 + f0;
       half8_t old = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -420,6 +434,11 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   c.raw_before[kRawParts] = 0;
   c.k_rows = p.k >> 5;                 // packed rows (32 dense k each)
   c.n_steps = (c.k_rows + 3) >> 2;     // 128 dense k per step
+  c.step0 = 0;
+  if (p.ksplit_steps) {                // this workgroup's share of the steps (the last share may be short, never empty)
+    c.step0 = blockIdx.z * p.ksplit_steps;
+    c.n_steps = min(p.ksplit_steps, c.n_steps - c.step0);
+  }
   c.qrow = p.m >> 1;
   c.mrow = p.m >> 2;
   // everything that depends on the delta: operand pointers and the request for this thread's scales
@@ -560,6 +579,35 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
     // the next pass over this group's tokens reuses s_rows / red
     if (t0 + gridDim.y * 16 * NT < count) lds_barrier();
   }
+}
+
+// Second pass of a K split across workgroups: out[row] = fp16(sum over splits, in the order of the splits, x scale).
+// One thread per 8 columns of a row; `rows_per_group` rows in a row share a delta (delta = group x delta_step).
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits, long rows, int m,
+                                                           const _Float16* __restrict__ scales, long scales_stride,
+                                                           int rows_per_group, int delta_step, _Float16* __restrict__ out,
+                                                           long out_stride) {
+  const long chunk = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int per_row = m >> 3;
+  const long row = chunk / per_row;
+  if (row >= rows) return;
+  const int f0 = (int)(chunk - row * per_row) * 8;
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] = 0.f;
+  for (int z = 0; z < splits; z++) {
+    const float* pp = partial + ((long)z * rows + row) * m + f0;
+    const float4_t a0 = *reinterpret_cast<const float4_t*>(pp);
+    const float4_t a1 = *reinterpret_cast<const float4_t*>(pp + 4);
+#pragma unroll
+    for (int i = 0; i < 4; i++) { v[i] += a0[i]; v[4 + i] += a1[i]; }
+  }
+  const long delta = (row / rows_per_group) * delta_step;
+  const half8_t sv = *reinterpret_cast<const half8_t*>(scales + delta * scales_stride + f0);
+  half8_t o;
+#pragma unroll
+  for (int i = 0; i < 8; i++) o[i] = scaled_sum_f16((_Float16)0, v[i], sv[i]);
+  *reinterpret_cast<half8_t*>(out + row * out_stride + f0) = o;
 }
 
 }  // namespace triteia_hip

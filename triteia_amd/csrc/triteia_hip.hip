@@ -137,7 +137,7 @@ void launch_one(const Sparse24Args& a, dim3 grid, hipStream_t st) {
 
 // `nt`: token tile class; `tsplit`: workgroups along y sharing one group's tokens (run-table form
 // only: plan tiles never exceed one pass, uniform groups are cut into chunks by the kernel).
-int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
+int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsplit = 1) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   if (tsplit < 1) tsplit = 1;
   if (tsplit > 65535) tsplit = 65535;
@@ -148,7 +148,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   // Only for uniform groups (matmul, bmm): the split of K among the wavefronts fixes the order of the
   // fp32 sums, and a routed token must have the same bits whatever the size of its batch.
   const bool uniform = !a.raw_indices && !a.tiles && !a.g_delta;
-  const bool one_per_cu = uniform && (nt == 1 || nt == 2) && (long)a.n_groups * cb_pad * tsplit <= 256;
+  const bool one_per_cu = uniform && zsplit == 1 && (nt == 1 || nt == 2) && (long)a.n_groups * cb_pad * tsplit <= 256;
   const int kw = knob_or(knobs().kw, one_per_cu ? 8 : 4);
   // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight (2 with
   // two), the 32-token kernel 2 per CU with two, the 64-token kernel 1 per CU with one.  Fused
@@ -158,7 +158,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   // launches that do not fill the GPU twice over (at most 512 workgroups) are bound by the latency
   // of each wave's chain of requests rather than by bandwidth: a second step in flight pays there
   // (5-12 % measured) while it costs time on full launches
-  const bool small = (long)a.n_groups * cb_pad * tsplit <= 512;
+  const bool small = (long)a.n_groups * cb_pad * tsplit * zsplit <= 512;
   const int depth = knob_or(knobs().depth, eager || kw == 8 ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1));
   if (eager && !(kw == 4 && ((nt == 1 && depth == 2) || (nt == 1 && depth == 1) || (nt == 2 && depth == 1) || (nt == 4 && depth == 1)))) {
     a.raw_static = 0;   // no eager build of this variant: route first, then request
@@ -175,7 +175,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st) {
   }
   const long units = (long)a.n_groups * cb_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
-  const dim3 grid((unsigned)units, (unsigned)tsplit);
+  const dim3 grid((unsigned)units, (unsigned)tsplit, (unsigned)zsplit);
 #define TRY(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
 #define TRY_EAGER(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_, true>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
   if (a.raw_indices && a.raw_static) {
@@ -278,28 +278,62 @@ bool wide_enabled() { return knobs().wide != 0; }
 constexpr long kWideMinUnits = 160;   // 4096 x 4096: 1024 tokens (128 tiles) 54.9 us wide against 46.5 us narrow, 1536 tokens (192) 60.8 against 71.1
 constexpr long kWide32MinUnits = 160, kWide32MaxUnits = 448;   // (32-token tile, 512-column group) units: see launch_uniform
 
-// `tokens` rows per group, `stride` rows between groups: the head of each group goes to the
-// 64-token kernel (full tiles, and a rest above half a tile), what is left to the narrow one.
-int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n_groups, hipStream_t st) {
-  a.n_groups = n_groups;
-  a.uniform_stride = stride;
-  a.delta_step = delta_step;
-  const long cgs = (a.m / 128 + 3) / 4;
+// ---- uniform groups (matmul, bmm): `tokens` rows per group.  Which kernel takes which rows is decided by
+// decide_uniform (a pure function of the shapes and the knobs, also behind triteia_hip_uniform_kernel) and carried
+// out by launch_uniform.
+enum UniformKind { kUniNarrow = 0, kUniWide32 = 32, kUniWide64 = 64, kUniTile256 = 256, kUniSplitK = 1000 };
+struct UniformSegment { int kind, first, count, ksplit; };
+struct UniformPlan { UniformSegment seg[3]; int n = 0; };
+
+// K split across workgroups for launches that leave most of the chip idle on a long K: (groups x column blocks x
+// token passes) well below the number of CUs and at least 64 steps of K.  Every workgroup takes 1 / ksplit of the K
+// steps and writes fp32 partial sums to a scratch buffer of the caller's; a second, tiny launch adds them in a fixed
+// order.  Returns the number of splits (1: none).  Measured (16 tokens, unsplit -> split in 4): 8192 x 8192 18.5 -> 14.2 us,
+// 11008 x 4096 22.5 -> 14.5 us.  A K of 4096 is too short to pay for the second launch (4096 x 4096: 11.4 -> 11.0 us in 4,
+// 12.4 in 8; with 64 tokens 11.0 -> 12.3; 4096 x 11008 12.5 -> 12.7), and so is a launch that has a workgroup per CU
+// already (8 matrices of 4096 x 4096 with one token each: 13.4 -> 16.5 us).
+constexpr long kSplitKMaxUnits = 64;    // launches of at most this many unsplit workgroups are split ...
+constexpr int kSplitKMinSteps = 64;     // ... if K has at least this many steps of 128 ...
+constexpr int kSplitKStepsPerSplit = 16;   // ... into shares of about this many steps
+int pick_ksplit(long tokens, long n_groups, int m, int k) {
+  if (!knobs().ksplit || tokens <= 0) return 1;
+  const long cb_pad = (m / 128 + 7) / 8 * 8;
+  const int nt = tokens <= 16 ? 1 : pick_nt_uniform(tokens, n_groups, m / 128);
+  const long units = n_groups * cb_pad * ((tokens + 16 * nt - 1) / (16 * nt));
+  const int n_steps = (k / 32 + 3) / 4;
+  if (knobs().ksplit > 1) return knobs().ksplit <= n_steps ? knobs().ksplit : n_steps;   // forced (tests, measurements)
+  if (units > kSplitKMaxUnits || n_steps < kSplitKMinSteps) return 1;
+  long ks = n_steps / kSplitKStepsPerSplit;
+  if (ks > 512 / units) ks = 512 / units;
+  if (ks > 16) ks = 16;
+  return ks < 2 ? 1 : (int)ks;
+}
+
+UniformPlan decide_uniform(int tokens, int stride, int n_groups, int m, int k, long x_stride, bool have_scratch) {
+  UniformPlan up;
+  auto add = [&](int kind, int first, int count, int ksplit = 1) { up.seg[up.n++] = UniformSegment{kind, first, count, ksplit}; };
+  const long cgs = (m / 128 + 3) / 4;
   int done = 0;
   bool ks64 = false;   // the whole launch goes to 64-token tiles on workgroups of eight wavefronts
   // (the wide kernels address activations with 32-bit byte offsets)
-  const bool x_below_4g = ((long)(n_groups - 1) * stride + tokens) * a.x_stride * 2 < (1L << 32);
+  const bool x_below_4g = ((long)(n_groups - 1) * stride + tokens) * x_stride * 2 < (1L << 32);
+  // Launches of a few dozen workgroups: K split across workgroups.
+  if (have_scratch) {
+    const int ks = pick_ksplit(tokens, n_groups, m, k);
+    if (ks > 1) {
+      add(kUniSplitK, 0, tokens, ks);
+      return up;
+    }
+  }
   // Groups of hundreds of tokens: 256-token x 256-column tiles whose wavefronts share the dequantised weights.
   if (knobs().tile256 && wide_enabled() && x_below_4g) {
-    const long ncp = (a.m / 128 + 1) / 2;
+    const long ncp = (m / 128 + 1) / 2;
     const long min_units = knob_or(knobs().tile256_min_units, kTile256MinUnits);
     int t = tokens / kT256Tokens * kT256Tokens;
     if (tokens - t >= kT256Tokens / 2 || min_units <= 1) t = tokens;     // a rest of half a tile and more is a tile
     const long units = (long)n_groups * ((t + kT256Tokens - 1) / kT256Tokens) * ncp;
     if (t > 0 && units >= min_units && units <= knob_or(knobs().tile256_max_units, kTile256MaxUnits)) {
-      a.uniform_first = 0;
-      a.uniform_count = t;
-      if (int e = launch_tile256(a, st)) return e;
+      add(kUniTile256, 0, t);
       done = t;
     }
   }
@@ -321,21 +355,19 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
     // are ahead while they make one workgroup per CU at most (4096 x 4096 with 1280 / 1536 tokens 49.7 -> 44.2,
     // 50.8 -> 46.0 us; 4096 x 11008 with 384 / 640 tokens 47.2 -> 43.0, 51.4 -> 46.0 us; 8192 x 8192 with 768 tokens 88.7 ->
     // 72.5 us; 8192 x 28672 with 192 tokens 89.4 -> 73.0 us)
-    ks64 = done == 0 && wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= kWideTokens &&
+    ks64 = done == 0 && wide_enabled() && k % 128 == 0 && x_below_4g && tokens >= kWideTokens &&
            units32 > knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits) &&
            (long)n_groups * ((tokens + kWideTokens - 1) / kWideTokens) * ((cgs + 7) / 8 * 8) <=
                knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits);
-    if (done == 0 && !ks64 && wide_enabled() && a.k % 128 == 0 && x_below_4g && tokens >= 32 &&
+    if (done == 0 && !ks64 && wide_enabled() && k % 128 == 0 && x_below_4g && tokens >= 32 &&
         units32 >= knob_or(knobs().wide32_min_units, kWide32MinUnits) &&
         units32 <= knob_or(knobs().wide32_max_units, kWide32MaxUnits)) {
-      a.uniform_first = 0;
-      a.uniform_count = tokens;
-      if (int e = launch_wide(a, st, 32)) return e;
+      add(kUniWide32, 0, tokens);
       done = tokens;
     }
   }
   int rest = tokens - done;
-  if (rest > 0 && wide_enabled() && a.k % 128 == 0 && x_below_4g &&
+  if (rest > 0 && wide_enabled() && k % 128 == 0 && x_below_4g &&
       (done > 0 ? rest >= kPlanWideMinRest
                 : ks64 || (long)n_groups * (rest / kWideTokens) * cgs >= knob_or(knobs().wide_min_units, kWideMinUnits))) {
     int t = rest / kWideTokens * kWideTokens;
@@ -345,17 +377,56 @@ int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n
     // 67.4 us).  Past one round the extra tile starts a round of its own (4104 tokens on 4096 x 4096: 88 -> 111 us).
     const bool one_round = (long)n_groups * (rest / kWideTokens + 1) * cgs <= 512;
     if (rest - t >= (one_round ? 1 : kPlanWideMinRest)) t = rest;
-    a.uniform_first = done;
-    a.uniform_count = t;
-    if (int e = launch_wide(a, st)) return e;
+    add(kUniWide64, done, t);
     done += t;
   }
   rest = tokens - done;
-  if (rest > 0) {
-    a.uniform_first = done;
-    a.uniform_count = rest;
-    const int nt = pick_nt_uniform(rest, n_groups, a.m / 128);
-    return launch_sparse24(a, nt, (rest + 16 * nt - 1) / (16 * nt), st);
+  if (rest > 0) add(kUniNarrow, done, rest);
+  return up;
+}
+
+// bytes of fp32 partial sums that a K split of this launch writes (0: the launch is not split)
+size_t uniform_scratch_bytes(int tokens, int n_groups, int m, int k) {
+  const int ks = pick_ksplit(tokens, n_groups, m, k);
+  return ks > 1 ? sizeof(float) * (size_t)ks * (size_t)n_groups * (size_t)tokens * (size_t)m : 0;
+}
+
+int launch_uniform(Sparse24Args a, int tokens, int stride, int delta_step, int n_groups, hipStream_t st,
+                   void* scratch = nullptr, size_t scratch_bytes = 0) {
+  a.n_groups = n_groups;
+  a.uniform_stride = stride;
+  a.delta_step = delta_step;
+  const bool have_scratch = scratch && stride == tokens && reinterpret_cast<uintptr_t>(scratch) % 16 == 0 &&
+                            scratch_bytes >= uniform_scratch_bytes(tokens, n_groups, a.m, a.k) &&
+                            uniform_scratch_bytes(tokens, n_groups, a.m, a.k) > 0;
+  const UniformPlan up = decide_uniform(tokens, stride, n_groups, a.m, a.k, a.x_stride, have_scratch);
+  for (int i = 0; i < up.n; i++) {
+    const UniformSegment& sg = up.seg[i];
+    a.uniform_first = sg.first;
+    a.uniform_count = sg.count;
+    int e = TRITEIA_HIP_OK;
+    if (sg.kind == kUniTile256) e = launch_tile256(a, st);
+    else if (sg.kind == kUniWide32) e = launch_wide(a, st, 32);
+    else if (sg.kind == kUniWide64) e = launch_wide(a, st);
+    else if (sg.kind == kUniSplitK) {
+      const int n_steps = (a.k / 32 + 3) / 4;
+      Sparse24Args b = a;
+      b.partial = static_cast<float*>(scratch);
+      b.partial_rows = (long)n_groups * tokens;
+      b.ksplit_steps = (n_steps + sg.ksplit - 1) / sg.ksplit;
+      const int splits = (n_steps + b.ksplit_steps - 1) / b.ksplit_steps;   // (every split has a step)
+      const int nt = sg.count <= 16 ? 1 : pick_nt_uniform(sg.count, n_groups, a.m / 128);
+      e = launch_sparse24(b, nt, (sg.count + 16 * nt - 1) / (16 * nt), st, splits);
+      if (e) return e;
+      const long chunks = b.partial_rows * (a.m / 8);
+      hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, b.partial, splits,
+                         b.partial_rows, a.m, a.scales, a.scales_stride, tokens, delta_step, a.out, a.out_stride);
+      e = check_launch("splitk_reduce_kernel");
+    } else {
+      const int nt = pick_nt_uniform(sg.count, n_groups, a.m / 128);
+      e = launch_sparse24(a, nt, (sg.count + 16 * nt - 1) / (16 * nt), st);
+    }
+    if (e) return e;
   }
   return TRITEIA_HIP_OK;
 }
@@ -414,8 +485,9 @@ int triteia_hip_mul_2_4(const void* A, const void* B, const void* meta, void* C,
   return launch_uniform(a, prob_n, prob_n, 0, 1, static_cast<hipStream_t>(stream));
 }
 
-int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
-                               int batch, int tokens, int prob_k, int dev, void* stream) {
+int triteia_hip_bmm_2_4_tokens_scratch(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
+                                       int batch, int tokens, int prob_k, void* scratch, size_t scratch_bytes, int dev,
+                                       void* stream) {
   if (int e = check_gemm_shape(prob_m, batch, prob_k, -1)) return e;
   if (tokens < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "bmm_2_4: tokens=%d", tokens);
   if (prob_m == 0 || batch == 0 || prob_k == 0 || tokens == 0) return TRITEIA_HIP_OK;
@@ -424,7 +496,37 @@ int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, v
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   Sparse24Args a;
   fill_weights(a, A, B, meta, C, s, prob_m, prob_k, batch);
-  return launch_uniform(a, tokens, tokens, 1, batch, static_cast<hipStream_t>(stream));
+  return launch_uniform(a, tokens, tokens, 1, batch, static_cast<hipStream_t>(stream), scratch, scratch_bytes);
+}
+
+int triteia_hip_bmm_2_4_tokens(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
+                               int batch, int tokens, int prob_k, int dev, void* stream) {
+  return triteia_hip_bmm_2_4_tokens_scratch(A, B, meta, C, s, prob_m, batch, tokens, prob_k, nullptr, 0, dev, stream);
+}
+
+size_t triteia_hip_bmm_scratch_bytes(int prob_m, int batch, int tokens, int prob_k) {
+  if (prob_m <= 0 || batch <= 0 || tokens <= 0 || prob_k <= 0 || prob_m % 128 != 0 || prob_k % 64 != 0) return 0;
+  return uniform_scratch_bytes(tokens, batch, prob_m, prob_k);
+}
+
+int triteia_hip_uniform_kernel(int prob_m, int batch, int tokens, int prob_k, int with_scratch) {
+  if (prob_m <= 0 || batch <= 0 || tokens <= 0 || prob_k <= 0 || prob_m % 128 != 0 || prob_k % 64 != 0) return -1;
+  const bool sc = with_scratch && uniform_scratch_bytes(tokens, batch, prob_m, prob_k) > 0;
+  const UniformPlan up = decide_uniform(tokens, tokens, batch, prob_m, prob_k, prob_k, sc);
+  if (up.n == 0) return -1;
+  // the segment that takes the most rows
+  int best = 0;
+  for (int i = 1; i < up.n; i++) if (up.seg[i].count > up.seg[best].count) best = i;
+  const UniformSegment& sg = up.seg[best];
+  if (sg.kind == kUniSplitK) return kUniSplitK + sg.ksplit;
+  if (sg.kind == kUniNarrow) return 0;
+  // 32- and 64-token tiles: + 1 when the launch runs on workgroups of eight wavefronts (halves of K)
+  const long cgs = (prob_m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
+  if (sg.kind == kUniWide32)
+    return 32 + ((long)batch * ((sg.count + 31) / 32) * cg_pad <= knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits) ? 1 : 0);
+  if (sg.kind == kUniWide64)
+    return 64 + ((long)batch * ((sg.count + 63) / 64) * cg_pad <= knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits) ? 1 : 0);
+  return sg.kind;
 }
 
 int triteia_hip_bmm_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m, int prob_n,
@@ -512,6 +614,16 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   return tiles * cgs >= knob_or(knobs().mid_min_units, kMidMinUnits);
 }
 constexpr int kFusedMaxTokens = 64 * kRawParts;   // kRawParts tokens per lane of a wavefront
+// The routed entry point routes inside the multiply kernel (one launch, no plan) or builds a plan first:
+static bool routed_eager_ok(int prob_n, int n_deltas) {
+  return n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && knobs().eager;
+}
+static bool routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
+  return prob_n <= knob_or(knobs().fused_max_tokens, kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
+         n_deltas <= (prob_n > 64 ? 32 : 64) && knobs().fused_route &&
+         !(prob_n >= 128 && ((!routed_eager_ok(prob_n, n_deltas) && mid_tiles(prob_n, n_deltas, prob_m, prob_k)) ||
+                             (long)prob_k * prob_m >= (1L << 27)));
+}
 static int plan_has_wide(int prob_n, int n_deltas) {
   const long groups = n_deltas < prob_n ? n_deltas : prob_n;
   return wide_enabled() && prob_n >= knobs().wide_min_batch && prob_n >= 8 * groups;
@@ -520,6 +632,11 @@ static int plan_has_wide(int prob_n, int n_deltas) {
 int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
   return mid_tiles(prob_n, n_deltas, prob_m, prob_k) ? triteia_hip_plan_tile_tokens(prob_n, n_deltas) : 0;
+}
+
+int triteia_hip_routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
+  if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
+  return routed_in_kernel(prob_n, n_deltas, prob_m, prob_k) ? 1 : 0;
 }
 
 int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
@@ -630,10 +747,8 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   // plan pays from 128 tokens on whatever the number of deltas, the plan launch being small against the kernel
   // and the wide kernels taking hot deltas: 8 / 4 deltas of 8192 x 28672 with 128 / 256 tokens 145 -> 130 /
   // 160 -> 122 us, while 8 or 16 deltas of 4096 x 11008 stay 8-12 % faster routed inside the kernel)
-  const bool eager_ok = n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && knobs().eager;
-  if (prob_n <= knob_or(knobs().fused_max_tokens, kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
-      n_deltas <= (prob_n > 64 ? 32 : 64) && knobs().fused_route &&
-      !(prob_n >= 128 && ((!eager_ok && mid_tiles(prob_n, n_deltas, prob_m, prob_k)) || (long)prob_k * prob_m >= (1L << 27)))) {
+  const bool eager_ok = routed_eager_ok(prob_n, n_deltas);
+  if (routed_in_kernel(prob_n, n_deltas, prob_m, prob_k)) {
     // small batch: the multiply kernel routes by itself, no plan, no workspace traffic
     if (!token_indices) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null indices");
     DeviceGuard g(dev);

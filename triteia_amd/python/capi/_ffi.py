@@ -26,6 +26,9 @@ SIGNATURES = {
     "triteia_hip_bmm_2_4": (_c_int, [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
     "triteia_hip_bmm_2_4_tokens": (_c_int, [_c_vp] * 5 + [_c_int] * 4 + [_c_int, _c_vp]),
     "triteia_hip_reload_env": (None, []),
+    "triteia_hip_bmm_2_4_tokens_scratch": (_c_int, [_c_vp] * 5 + [_c_int] * 4 + [_c_vp, _c_sz, _c_int, _c_vp]),
+    "triteia_hip_bmm_scratch_bytes": (_c_sz, [_c_int] * 4),
+    "triteia_hip_uniform_kernel": (_c_int, [_c_int] * 5),
     "triteia_hip_sbmm_2_4": (_c_int, [_c_vp] * 8 + [_c_int] * 4 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 4),
     "triteia_hip_sbmm_2_4_bounded": (_c_int, [_c_vp] * 8 + [_c_int] * 4 + [_c_vp, _c_int, _c_int, _c_vp] + [_c_int] * 5),
     "triteia_hip_sbmm_2_4_routed": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_vp, _c_sz, _c_int, _c_int, _c_vp]),
@@ -34,6 +37,7 @@ SIGNATURES = {
     "triteia_hip_sbmm_2_4_planned": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_int, _c_vp]),
     "triteia_hip_sbmm_routed_workspace_bytes": (_c_sz, [_c_int, _c_int]),
     "triteia_hip_plan_tile_tokens": (_c_int, [_c_int, _c_int]),
+    "triteia_hip_routed_in_kernel": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
     "triteia_hip_planned_tile_kernel": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
     "triteia_hip_route_plan": (_c_int, [_c_vp, _c_int, _c_int, _c_int, _c_vp, _c_sz, _c_int, _c_vp]),
     "triteia_hip_bgmv": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_float, _c_int, _c_vp]),
@@ -104,6 +108,21 @@ def require_gpu(**tensors):
 def require_dtype(t, dtype, name):
     if t.dtype != dtype:
         raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
+
+
+_SPLIT_SCRATCH = {}
+
+
+def split_scratch(nbytes: int, device) -> torch.Tensor:
+    """Scratch for the K split of small matmul / bmm launches (fp32 partial sums): one buffer per device and
+    stream, grown on demand, so that calls on different streams never share one."""
+    dev = torch.device(device)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    buf = _SPLIT_SCRATCH.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 4 << 20), dtype=torch.uint8, device=dev)
+        _SPLIT_SCRATCH[key] = buf
+    return buf
 
 
 _LOCK_WORKSPACES = {}

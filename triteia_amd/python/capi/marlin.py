@@ -56,9 +56,19 @@ def mul_2_4(A, B, meta, C, s, workspace, thread_k=-1, thread_m=-1, sms=-1, max_p
         raise RuntimeError(f"workspace must be of size at least {prob_m // 128 * max_par}.")
     if groupsize == -1 and prob_m % 128 == 0 and prob_k % 64 == 0:
         _check_packed(B, meta, s, prob_m, prob_k)
-    err = _ffi.lib().triteia_hip_mul_2_4(
-        _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), prob_m, prob_n, prob_k,
-        _ffi.ptr(workspace), groupsize, _ffi.device_index(A), _ffi.stream_of(A), thread_k, thread_m, sms, max_par)
+    lib = _ffi.lib()
+    split = lib.triteia_hip_bmm_scratch_bytes(prob_m, 1, prob_n, prob_k) if groupsize == -1 else 0
+    if split:
+        # a launch of few workgroups: K is split across workgroups through a scratch buffer of this binding's (the
+        # reference's lock workspace is too small for partial sums); same entry point as bmm with one matrix
+        scratch = _ffi.split_scratch(split, A.device)
+        err = lib.triteia_hip_bmm_2_4_tokens_scratch(
+            _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), prob_m, 1, prob_n, prob_k,
+            _ffi.ptr(scratch), scratch.numel(), _ffi.device_index(A), _ffi.stream_of(A))
+    else:
+        err = lib.triteia_hip_mul_2_4(
+            _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), prob_m, prob_n, prob_k,
+            _ffi.ptr(workspace), groupsize, _ffi.device_index(A), _ffi.stream_of(A), thread_k, thread_m, sms, max_par)
     _raise(err, prob_m, prob_n, prob_k, thread_k, thread_m, groupsize)
 
 
@@ -78,7 +88,14 @@ def bmm_2_4(A, B, meta, C, s, workspace, thread_k=-1, thread_m=-1, sms=-1, max_p
         _raise(_ffi.ERR_KERN_SHAPE, prob_m, batch, prob_k, thread_k, thread_m, groupsize)
     if prob_m % 128 == 0 and prob_k % 64 == 0:
         _check_packed(B, meta, s, prob_m, prob_k, lead=(batch,))
-    if tokens == 1:
+    lib = _ffi.lib()
+    split = lib.triteia_hip_bmm_scratch_bytes(prob_m, batch, tokens, prob_k) if prob_m % 128 == 0 and prob_k % 64 == 0 else 0
+    if split:
+        scratch = _ffi.split_scratch(split, A.device)
+        err = lib.triteia_hip_bmm_2_4_tokens_scratch(
+            _ffi.ptr(A), _ffi.ptr(B), _ffi.ptr(meta), _ffi.ptr(C), _ffi.ptr(s), prob_m, batch, tokens, prob_k,
+            _ffi.ptr(scratch), scratch.numel(), _ffi.device_index(A), _ffi.stream_of(A))
+    elif tokens == 1:
         # the reference's own case and argument list (triteia_nm_bmm.cu:760-764)
         if workspace.numel() < prob_m // 128 * max_par:
             raise RuntimeError(f"workspace must be of size at least {prob_m // 128 * max_par}.")
