@@ -138,7 +138,7 @@ TRITEIA_HIP_API int triteia_hip_sbmm_2_4_bounded(const void* A, const void* B, c
  * workspace: >= triteia_hip_sbmm_routed_workspace_bytes(prob_n, n_deltas) bytes
  * of device memory, contents irrelevant on entry, overwritten (batches of at most 64
  * tokens over at most 64 deltas are always routed inside the multiply kernel and leave it
- * untouched; so are most batches of up to 256 tokens over at most 32 deltas, but not all:
+ * untouched; so are most batches of up to 256 tokens over at most 16 deltas, but not all:
  * pass the workspace for every batch above 64 tokens).
  * n_deltas <= 8192. */
 TRITEIA_HIP_API int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, void* C, const void* s,

@@ -470,19 +470,23 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
       if (grp >= p.n_deltas) return;
       delta = grp;
       bind_delta(delta);
+      // (only the workgroup that takes a group's first tokens: the others of a launch that splits a group's tokens over
+      // blockIdx.y mostly find nothing to do, and a prefetched step each would be traffic for nothing)
+      if (blockIdx.y == 0) {
 #pragma unroll
-      for (int j = 0; j < NPRE; j++) {
-        const int st = c.wave + j * KW;              // this wave's j-th step (beyond the end of K: loads go unused)
-        int ps = st + c.rot;
-        if (ps >= c.n_steps) ps -= c.n_steps;
-        if (st >= c.n_steps) ps = 0;
-        const int tr = min((ps << 2) + c.q, c.k_rows - 1);
-        const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
-        const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
+        for (int j = 0; j < NPRE; j++) {
+          const int st = c.wave + j * KW;              // this wave's j-th step (beyond the end of K: loads go unused)
+          int ps = st + c.rot;
+          if (ps >= c.n_steps) ps -= c.n_steps;
+          if (st >= c.n_steps) ps = 0;
+          const int tr = min((ps << 2) + c.q, c.k_rows - 1);
+          const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
+          const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
 #pragma unroll
-        for (int a = 0; a < 4; a++) pre[j].wq[a] = wp[a];
-        pre[j].mt[0] = mp[0];
-        pre[j].mt[1] = mp[8];
+          for (int a = 0; a < 4; a++) pre[j].wq[a] = wp[a];
+          pre[j].mt[0] = mp[0];
+          pre[j].mt[1] = mp[8];
+        }
       }
       // nothing that needs the indices may be scheduled (with its wait) ahead of these requests
       __builtin_amdgcn_sched_barrier(0);
@@ -560,7 +564,7 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   bool first_pass = true;
   for (int t0 = blockIdx.y * 16 * NT; t0 < count; t0 += gridDim.y * 16 * NT) {
     const int cnt = min(count - t0, 16 * NT);
-    if (EAGER && first_pass) {
+    if (EAGER && first_pass && blockIdx.y == 0) {
       if (NT == 1 || cnt <= 16) {
         tile_pass<1, KW, (NT == 1 ? DEPTH : 2), NPRE>(p, c, start + t0, cnt, red, s_rows, pre);
       } else if (NT == 2 || cnt <= 32) {

@@ -57,7 +57,7 @@ struct Knobs {
   int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
-  int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset;
+  int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
   int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1;
 };
@@ -73,7 +73,7 @@ void read_knobs() {
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
       {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
-      {"MID_MIN_UNITS", &k.mid_min_units}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
+      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
       {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
       {"KSPLIT", &k.ksplit},
   };
@@ -113,6 +113,10 @@ int pick_nt(long tokens, long groups) {
   // with more tokens some delta of a skewed batch is always hot and 32-token tiles win
   if (tokens <= 64 && tokens <= 4 * groups) return 1;
   if (tokens <= 24 * groups) return 2;   // typical group well under 32 tokens
+  // few tiles in all (64-token tiles: one per 64 tokens and a last one per group): 32-token tiles make twice as
+  // many workgroups of them (4 deltas of 4096 x 4096 with 1024 tokens: 55 -> 46 us; 16 deltas: 66 -> 61.5 us with 1024
+  // tokens, 86.6 -> 82.1 with 2048; 32 deltas of 11008 x 4096 with 1024: 184 -> 156 us)
+  if (tokens / 64 + groups <= 48) return 2;
   return 4;
 }
 
@@ -266,11 +270,12 @@ int launch_tile256(const Sparse24Args& a, hipStream_t st) {
   hipLaunchKernelGGL(sparse24_tile256_kernel, dim3((unsigned)units), dim3(512), kT256LdsBytes, st, a);
   return check_launch("sparse24_tile256_kernel");
 }
-// (token tile, column pair) units for which a uniform launch takes this kernel: launches of about one round of workgroups
-// (one per CU).  Measured against 64-token tiles: 4096 tokens on 4096 x 4096 (256 units) 89.1 against 95.8 us, on
-// 8192 x 8192 (512 units) 290 against 294 us; 4096 x 11008 (688 units) 228 against 227 us; 8192 x 28672 (1792 units)
-// 994 against 950 us; 2048 tokens on 4096 x 4096 (128 units: half the CUs idle) 72 against 55 us.
-constexpr long kTile256MinUnits = 192, kTile256MaxUnits = 512;
+// (token tile, column pair) units for which a uniform launch takes this kernel: launches of one round of workgroups
+// (one per CU) that fill most of the chip.  Measured against 64-token tiles: 4096 tokens on 4096 x 4096 (256 units) 89.1
+// against 95.8 us (82.8 against 83.4 on another box), on 8192 x 8192 (512 units) 290 against 294 us; 4096 x 11008
+// (688 units) 228 against 227 us; 8192 x 28672 (1792 units) 994 against 950 us; 2048 tokens on 4096 x 11008 (344 units:
+// a second round of a third of the chip) 139 against 116 us; on 4096 x 4096 (128 units: half the CUs idle) 72 against 55 us.
+constexpr long kTile256MinUnits = 192, kTile256MaxUnits = 256;
 
 // The wide kernel pays off when there are enough tiles to occupy the GPU; below that the narrow
 // kernel's smaller units win.  Knob `wide` = 0 disables it; `wide_min_units` moves the threshold.
@@ -595,7 +600,8 @@ constexpr int kPlanWideMinUnits = 150;
 // about 450 (tile, 512-column group) units (cfg3 at 128 / 256 / 512 tokens 66.6 -> 62.7, 97 -> 88, 133 -> 126.5 us;
 // 8 deltas of 8192 x 28672 with 96 tokens 142 -> 128.5 us), slower below (16 deltas of 4096 x 4096 with 256 tokens
 // 24.9 -> 42.4 us).  The host only has the upper bound on the tiles; 600 on that bound separates the measured cases.
-constexpr int kMidMinUnits = 600;
+constexpr int kMidMinUnits = 480;
+constexpr int kMidNarrowMinUnits = 280, kMidNarrowMinUnits64 = 150, kMidNarrowMinTokens = 768, kMidNarrowMaxTokens = 2048;
 static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   const int tile = triteia_hip_plan_tile_tokens(prob_n, n_deltas);
   // (64-token plans as well, on the 64-token build, where K is short: cfg3 at 1024 / 2048 tokens 196 -> 170 /
@@ -605,12 +611,20 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (prob_k % 128 != 0 || (long)prob_n * prob_k * 2 >= (1L << 32)) return false;   // whole K steps, 32-bit activation offsets
   const long tiles = (n_deltas < prob_n ? n_deltas : prob_n) + prob_n / tile;
   // (and only with a few tokens per tile at least: with two or three the shared activation tile saves nothing
-  // and the longer workgroups cost: 200 tokens over 65 of 512 resident deltas of 4096 x 11008 212 -> 238 us)
-  if (2 * prob_n < 7 * tiles) return false;
-  // (and a layer of 16 column groups at least: on m = 4096 it is even at best, 64 deltas with 8 tokens each 80 us
-  // both ways, and loses with few tokens per tile, 128 deltas with 6 each 146 -> 164 us)
+  // and the longer workgroups cost: 200 tokens over 65 of 512 resident deltas of 4096 x 11008 212 -> 238 us; at 3.6 per
+  // tile on the bound, 128 tokens over 32 deltas of 4096 x 11008, it depends on the routing: 82 -> 92 us under Zipf(1.0),
+  // 76 -> 66 us under Zipf(1.2))
+  if (2 * (long)prob_n < (long)knobs().mid_min_half_tokens * tiles) return false;
   const long cgs = (prob_m / 128 + 3) / 4;
-  if (cgs < knobs().mid_min_column_groups) return false;
+  if (cgs < knobs().mid_min_column_groups) {
+    // A layer of fewer than 16 column groups (m = 4096): with few tokens per tile it is even at best (64 deltas with 8
+    // tokens each 80 us both ways) or loses (128 deltas with 6 each 146 -> 164 us); with a thousand tokens in tiles
+    // that are mostly full it wins (4 / 16 / 64 deltas of 4096 x 4096, 1024 tokens: 65 -> 56, 72 -> 65, 107 -> 103 us),
+    // as long as the launch has work for the chip (16 deltas with 512 tokens, 256 units on the bound: 45 -> 50 us) and
+    // the batch is not one whose hot deltas fill the chip with 64-token tiles of their own (16 deltas, 4096 tokens:
+    // 134 -> 153 us).
+    return knobs().mid_narrow && prob_n >= kMidNarrowMinTokens && prob_n < kMidNarrowMaxTokens && tiles * cgs >= (tile == 64 ? kMidNarrowMinUnits64 : kMidNarrowMinUnits);
+  }
   return tiles * cgs >= knob_or(knobs().mid_min_units, kMidMinUnits);
 }
 constexpr int kFusedMaxTokens = 64 * kRawParts;   // kRawParts tokens per lane of a wavefront
@@ -620,7 +634,7 @@ static bool routed_eager_ok(int prob_n, int n_deltas) {
 }
 static bool routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   return prob_n <= knob_or(knobs().fused_max_tokens, kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
-         n_deltas <= (prob_n > 64 ? 32 : 64) && knobs().fused_route &&
+         n_deltas <= (prob_n > 64 ? 16 : 64) && knobs().fused_route &&
          !(prob_n >= 128 && ((!routed_eager_ok(prob_n, n_deltas) && mid_tiles(prob_n, n_deltas, prob_m, prob_k)) ||
                              (long)prob_k * prob_m >= (1L << 27)));
 }
@@ -739,8 +753,8 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
   if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: accumulate=%d", accumulate);
   if (prob_m == 0 || prob_n == 0 || prob_k == 0 || n_deltas == 0) return TRITEIA_HIP_OK;
   if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null tensor pointer");
-  // (above 64 tokens only for at most 32 deltas: with 64 deltas of 8192 x 28672 under a skewed routing the
-  // workgroups of the deltas without tokens make this form 1-2 % slower than a plan, which lists none)
+  // (above 64 tokens only for at most 16 deltas, whose weights can be requested ahead of the routing: with 32 deltas of
+  // 11008 x 4096 and 256 tokens a plan is 10-15 % faster, with 64 deltas of 8192 x 28672 under a skewed routing 1-2 %)
   // (and from 128 tokens on, a batch whose deltas' weights are not requested ahead of the routing is better
   // off with a plan where the plan's tiles go to the 32-token wide kernel: 32 deltas of 4096 x 11008,
   // 128 / 256 tokens: 69 -> 65.5 / 96 -> 89.5 us including the plan; on very large layers (k x m >= 2^27) a
@@ -771,7 +785,13 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
       a.raw_static = 1;
       a.n_groups = n_deltas;
     }
-    return launch_sparse24(a, nt, 1, static_cast<hipStream_t>(stream));
+    // Above 64 tokens a delta may hold several passes' worth of tokens (a skewed routing, or few deltas): its passes are
+    // spread over up to four workgroups instead of running one after the other in one (4 deltas of 4096 x 4096 with 256
+    // tokens: 44 -> 21 us; the workgroups that find no pass of their own leave after the routing).
+    // (from 33 tokens on already where the weights are not requested ahead of the routing, i.e. where a workgroup without
+    // a pass costs nothing but its routing: 64 tokens under Zipf(1.2) over 32 deltas of 11008 x 4096, 70 -> 64 us)
+    const long tsplit = prob_n <= (eager_ok ? 64 : 32) ? 1 : (prob_n <= 128 ? 2 : 4);
+    return launch_sparse24(a, nt, tsplit, static_cast<hipStream_t>(stream));
   }
   if (int e = triteia_hip_route_plan(token_indices, index_offset, n_deltas, prob_n, workspace, workspace_bytes, dev, stream))
     return e;
