@@ -214,6 +214,10 @@ TRITEIA_HIP_API int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, c
  * and min(h_in, h_out) <= 128, else ERR_KERN_SHAPE ("No suitable kernel"). */
 TRITEIA_HIP_API int triteia_hip_bgmv(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
                      int num_layers, int layer_idx, float scale, int dev, void* stream);
+/* The same for bf16 tensors (Y, X, W): the reference instantiates bgmv_kernel for nv_half and nv_bfloat16
+ * (triteia/csrc/ops/bgmv_all.cu:4-5) and dispatches on the tensors' dtype (ops.cpp:199-214). */
+TRITEIA_HIP_API int triteia_hip_bgmv_bf16(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                          int num_layers, int layer_idx, float scale, int dev, void* stream);
 
 /* SGMV: y[s[i] : s[i+1]] += x[s[i] : s[i+1]] @ W_i, W_i = (fp16*)w_ptrs[i] +
  * layer_idx * d_in * d_out, row-major [d_in, d_out]; s int32 [num_problems+1].
@@ -223,6 +227,10 @@ TRITEIA_HIP_API int triteia_hip_bgmv(void* Y, const void* X, const void* W, cons
 TRITEIA_HIP_API int triteia_hip_sgmv(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
                      int d_out, int layer_idx, int dev, void* stream);
 TRITEIA_HIP_API size_t triteia_hip_sgmv_tmp_size(int num_problems); /* reference: sgmv_tmp_size, sgmv.cuh:48-52 */
+/* The same for bf16 tensors (y, x and the matrices behind w_ptrs): sgmv<nv_bfloat16> (triteia/csrc/ops/sgmv.cu:10,
+ * dispatched on x's dtype, ops.cpp:132-143). */
+TRITEIA_HIP_API int triteia_hip_sgmv_bf16(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
+                          int d_out, int layer_idx, int dev, void* stream);
 
 /* Routed SGMV on a routing plan made by triteia_hip_route_plan: for every group
  * g (adapter a = g_delta[g]) and every listed row t:
@@ -233,6 +241,11 @@ TRITEIA_HIP_API size_t triteia_hip_sgmv_tmp_size(int num_problems); /* reference
 TRITEIA_HIP_API int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
                             int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
                             int dev, void* stream);
+
+/* The same for bf16 tensors (y, x, w_base). */
+TRITEIA_HIP_API int triteia_hip_sgmv_routed_bf16(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
+                                 int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
+                                 int dev, void* stream);
 
 #ifdef __cplusplus
 }

@@ -342,22 +342,32 @@ def sbmm_4bit_2_4(qweights, xs, metas, ss, indices, base_weight=None) -> np.ndar
     return y
 
 
-def lora(weights_A, weights_B, x, indices, base_weight=None, scale=1.0) -> np.ndarray:
+def round_bf16(a) -> np.ndarray:
+    """Round to the nearest bfloat16 (ties to even), returned as float64: the upper 16 bits of the fp32 pattern."""
+    bits = np.asarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+    return bits.astype(np.uint32).view(np.float32).astype(np.float64)
+
+
+def lora(weights_A, weights_B, x, indices, base_weight=None, scale=1.0, intermediate="f16") -> np.ndarray:
     """y[t] = base(x[t]) + scale * fp16(x[t] @ A_i) @ B_i for i = indices[t] >= 0 (lora.py:4-20).
 
-    The rank-r intermediate is rounded to fp16 as every reference variant does
-    (torch fp16 matmul, punica.py:27,64 fp16 temporaries).
+    The rank-r intermediate is rounded to the tensors' type as every reference variant does
+    (torch matmul in that type, punica.py:27,64 temporaries of x's dtype): fp16, or bf16 for the
+    reference's bfloat16 instantiation (bgmv_all.cu:5, sgmv.cu:10; inputs then come as float32
+    arrays holding bf16 values).
     """
+    rnd = round_bf16 if intermediate == "bf16" else (lambda a: np.asarray(a).astype(np.float16).astype(np.float64))
     T = x.shape[0]
     m = weights_B.shape[2]
     x64 = x.astype(np.float64)
     y = np.zeros((T, m), dtype=np.float64)
     if base_weight is not None:
-        y = (x64 @ base_weight.astype(np.float64).T).astype(np.float16).astype(np.float64)
+        y = rnd(x64 @ base_weight.astype(np.float64).T)
     for t in range(T):
         i = int(indices[t])
         if i >= 0:
-            v = (x64[t] @ weights_A[i].astype(np.float64)).astype(np.float16).astype(np.float64)
+            v = rnd(x64[t] @ weights_A[i].astype(np.float64))
             y[t] += scale * (v @ weights_B[i].astype(np.float64))
     return y
 

@@ -684,6 +684,33 @@ def test_lora_ops(ops, T, M, k, m, r, seed):
     check_close(ops.lora_sgmv_routed(gA, gB, gx2, gi2), ref2, what="lora_sgmv_routed unsorted")
 
 
+@pytest.mark.parametrize("T,M,k,m,r,seed", [
+    (10, 5, 768, 256, 64, 161), (33, 4, 512, 1024, 16, 162), (71, 3, 512, 520, 24, 163), (41, 2, 1024, 512, 128, 164),
+])
+def test_lora_ops_bf16(ops, T, M, k, m, r, seed):
+    """The bfloat16 instantiation of BGMV / SGMV (the reference builds both element types: bgmv_all.cu:4-5,
+    sgmv.cu:10).  bf16 keeps 8 significant bits: one rounding of an output is up to 2^-9 relative (1.1e-3 rms),
+    and the rank-r intermediate, rounded to bf16 as well, can fall on the other side of a rounding boundary when
+    the fp32 sums are taken in another order; the bound here is 1e-2 relative Frobenius error."""
+    say(f"lora bf16 T={T} M={M} k={k} m={m} r={r} seed={seed}")
+    rng = np.random.default_rng(seed)
+    A = orc.round_bf16(rng.standard_normal((M, k, r)) * 0.1).astype(np.float32)
+    B = orc.round_bf16(rng.standard_normal((M, r, m)) * 0.1).astype(np.float32)
+    x = orc.round_bf16(rng.standard_normal((T, k))).astype(np.float32)
+    idx = np.sort(rng.integers(-1, M, size=T)).astype(np.int32)
+    ref = orc.lora(A, B, x, idx, intermediate="bf16")
+    gA, gB, gx = (torch.from_numpy(a).to(DEV).to(torch.bfloat16) for a in (A, B, x))
+    gi = torch.from_numpy(idx).to(DEV)
+    for name in ("lora_bgmv", "lora_sgmv", "lora_sgmv_routed", "lora_forloop"):
+        out = getattr(ops, name)(gA, gB, gx, gi)
+        torch.cuda.synchronize()
+        assert out.dtype == torch.bfloat16
+        check_close(out, ref, tol=1e-2, what=name + " bf16")
+        assert bool((out[torch.from_numpy(idx < 0).to(DEV)] == 0).all())
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        ops.lora_sgmv_routed(gA.half(), gB, gx, gi)          # mixed element types are refused
+
+
 @pytest.mark.parametrize("T,M,N,m,k,r,seed", [
     (10, 5, 5, 768, 768, 8, 71), (10, 5, 5, 768, 768, 64, 72),          # tests/ops/test_ldmm.py:103
     (128, 2, 3, 4096, 2048, 16, 73), (128, 16, 16, 1024, 1024, 32, 74),

@@ -275,3 +275,28 @@ def test_ops_against_python_loops():
             assert np.allclose(ym[t], orc.lora(A, B, x[t:t + 1], np.array([i]))[0])
         else:
             assert np.allclose(ym[t], x[t].astype(np.float64) @ dense[i - M].astype(np.float64))
+
+
+def test_round_bf16_against_the_torch_conversion():
+    """The oracle's bfloat16 rounding (for the LoRA ops' bf16 instantiation) against torch's own conversion,
+    ties included (0x3F808000 lies halfway between two bf16 values and goes to the even one)."""
+    import torch
+    rng = np.random.default_rng(5)
+    a = np.concatenate([rng.standard_normal(20000) * 7, rng.standard_normal(2000) * 1e-3,
+                        np.array([0x3F808000, 0x3F818000, 0x3F807FFF, 0x3F808001, 0xBF808000], dtype=np.uint32).view(np.float32)])
+    want = torch.from_numpy(a.astype(np.float32)).to(torch.bfloat16).double().numpy()
+    assert np.array_equal(orc.round_bf16(a), want)
+    # and the lora restatement with that rounding against a plain loop
+    A = orc.round_bf16(rng.standard_normal((2, 16, 8))).astype(np.float32)
+    B = orc.round_bf16(rng.standard_normal((2, 8, 24))).astype(np.float32)
+    x = orc.round_bf16(rng.standard_normal((5, 16))).astype(np.float32)
+    idx = np.array([1, -1, 0, 1, 0])
+    got = orc.lora(A, B, x, idx, intermediate="bf16")
+    for t in range(5):
+        if idx[t] < 0:
+            assert not got[t].any()
+            continue
+        v = [float(torch.tensor(sum(float(x[t, i]) * float(A[idx[t], i, j]) for i in range(16)), dtype=torch.float32).to(torch.bfloat16))
+             for j in range(8)]
+        want_row = [sum(v[j] * float(B[idx[t], j, c]) for j in range(8)) for c in range(24)]
+        assert np.allclose(got[t], want_row, rtol=1e-12, atol=1e-12)

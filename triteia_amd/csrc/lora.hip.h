@@ -1,6 +1,7 @@
 // LoRA matrix-vector kernels for gfx950: BGMV (one adapter per token) and SGMV
-// (one adapter per segment / group of tokens).  fp16 in, fp32 accumulate,
-// fp16 read-modify-write of y.
+// (one adapter per segment / group of tokens).  Element type T = fp16 or bf16 (the reference
+// instantiates both: triteia/csrc/ops/bgmv_all.cu:4-5, sgmv.cu:10), fp32 accumulate,
+// read-modify-write of y in T.
 //
 // Semantics follow the reference:
 //   BGMV  Y[b, j] += scale * sum_i W[idx_b * L + layer][j][i] * X[b][i]
@@ -20,8 +21,8 @@
 
 namespace triteia_hip {
 
-typedef _Float16 lhalf8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 lhalf2_t __attribute__((ext_vector_type(2)));
+template <class T> using lvec8 = T __attribute__((ext_vector_type(8)));
+template <class T> using lvec2 = T __attribute__((ext_vector_type(2)));
 
 constexpr int kLoraMaxNarrow = 128;
 
@@ -42,33 +43,35 @@ __device__ __forceinline__ float wave_sum(float v) {
 // ---------------------------------------------------------------- BGMV ----
 
 // wide -> narrow: grid (B), block 256.  Wave w computes outputs j = w, w+4, ...
-__global__ __launch_bounds__(256) void bgmv_shrink_kernel(_Float16* __restrict__ Y, const _Float16* __restrict__ X,
-                                                         const _Float16* __restrict__ W,
+template <class T>
+__global__ __launch_bounds__(256) void bgmv_shrink_kernel(T* __restrict__ Y, const T* __restrict__ X,
+                                                         const T* __restrict__ W,
                                                          const long long* __restrict__ indices, int h_in, int h_out,
                                                          long num_layers, long layer_idx, float scale) {
   const int b = blockIdx.x;
   const long idx = indices[b];
   if (idx < 0) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const _Float16* w = W + (idx * num_layers + layer_idx) * (long)h_out * h_in;
-  const _Float16* x = X + (long)b * h_in;
+  const T* w = W + (idx * num_layers + layer_idx) * (long)h_out * h_in;
+  const T* x = X + (long)b * h_in;
   for (int j = wave; j < h_out; j += 4) {
-    const _Float16* wj = w + (long)j * h_in;
+    const T* wj = w + (long)j * h_in;
     float acc = 0.f;
     for (int i = lane * 8; i < h_in; i += 512) {
-      const lhalf8_t wv = *reinterpret_cast<const lhalf8_t*>(wj + i);
-      const lhalf8_t xv = *reinterpret_cast<const lhalf8_t*>(x + i);
+      const lvec8<T> wv = *reinterpret_cast<const lvec8<T>*>(wj + i);
+      const lvec8<T> xv = *reinterpret_cast<const lvec8<T>*>(x + i);
 #pragma unroll
       for (int e = 0; e < 8; e++) acc += (float)wv[e] * (float)xv[e];
     }
     acc = wave_sum(acc) * scale;
-    if (lane == 0) Y[(long)b * h_out + j] = (_Float16)((float)Y[(long)b * h_out + j] + acc);
+    if (lane == 0) Y[(long)b * h_out + j] = (T)((float)Y[(long)b * h_out + j] + acc);
   }
 }
 
 // narrow -> wide: grid (ceil(h_out / 256), B), block 256, one output per thread
-__global__ __launch_bounds__(256) void bgmv_expand_kernel(_Float16* __restrict__ Y, const _Float16* __restrict__ X,
-                                                         const _Float16* __restrict__ W,
+template <class T>
+__global__ __launch_bounds__(256) void bgmv_expand_kernel(T* __restrict__ Y, const T* __restrict__ X,
+                                                         const T* __restrict__ W,
                                                          const long long* __restrict__ indices, int h_in, int h_out,
                                                          long num_layers, long layer_idx, float scale) {
   __shared__ float xs[kLoraMaxNarrow];
@@ -79,28 +82,29 @@ __global__ __launch_bounds__(256) void bgmv_expand_kernel(_Float16* __restrict__
   __syncthreads();
   const int j = blockIdx.x * 256 + threadIdx.x;
   if (j >= h_out) return;
-  const _Float16* wj = W + ((idx * num_layers + layer_idx) * (long)h_out + j) * h_in;
+  const T* wj = W + ((idx * num_layers + layer_idx) * (long)h_out + j) * h_in;
   float acc = 0.f;
   for (int i = 0; i < h_in; i += 8) {
-    const lhalf8_t wv = *reinterpret_cast<const lhalf8_t*>(wj + i);
+    const lvec8<T> wv = *reinterpret_cast<const lvec8<T>*>(wj + i);
 #pragma unroll
     for (int e = 0; e < 8; e++) acc += (float)wv[e] * xs[i + e];
   }
-  _Float16* yp = Y + (long)b * h_out + j;
-  *yp = (_Float16)((float)*yp + acc * scale);
+  T* yp = Y + (long)b * h_out + j;
+  *yp = (T)((float)*yp + acc * scale);
 }
 
 // ---------------------------------------------------------------- SGMV ----
 
-struct SgmvArgs {
-  _Float16* y;
+template <class T>
+struct SgmvArgsT {
+  T* y;
   long y_stride;
-  const _Float16* x;
+  const T* x;
   long x_stride;
   int d_in, d_out;
   // weights: pointer per group (w_ptrs) or w_base + adapter * w_stride; layer_off added to either
   const long long* w_ptrs;
-  const _Float16* w_base;
+  const T* w_base;
   long w_stride;
   long layer_off;
   // groups: indptr `seg` (group g = rows seg[g]..seg[g+1], adapter g), or the
@@ -114,12 +118,16 @@ struct SgmvArgs {
   float scale;
 };
 
-struct SgmvGroup {
-  const _Float16* w;
+using SgmvArgs = SgmvArgsT<_Float16>;
+
+template <class T>
+struct SgmvGroupT {
+  const T* w;
   int start, count;
 };
 
-__device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* out) {
+template <class T>
+__device__ __forceinline__ bool sgmv_group(const SgmvArgsT<T>& a, int g, SgmvGroupT<T>* out) {
   int adapter, n = a.n_groups;
   if (a.seg) {
     adapter = g;
@@ -136,19 +144,20 @@ __device__ __forceinline__ bool sgmv_group(const SgmvArgs& a, int g, SgmvGroup* 
     out->count = d.z;
   }
   if (out->count <= 0 || adapter < 0 || adapter >= a.n_adapters) return false;
-  const _Float16* base = a.w_ptrs ? reinterpret_cast<const _Float16*>(a.w_ptrs[adapter]) : a.w_base + adapter * a.w_stride;
+  const T* base = a.w_ptrs ? reinterpret_cast<const T*>(a.w_ptrs[adapter]) : a.w_base + adapter * a.w_stride;
   out->w = base + a.layer_off;
   return true;
 }
 
-__device__ __forceinline__ int sgmv_row(const SgmvArgs& a, int i) { return a.perm ? a.perm[i] : i; }
+template <class T>
+__device__ __forceinline__ int sgmv_row(const SgmvArgsT<T>& a, int i) { return a.perm ? a.perm[i] : i; }
 
 // The rows of R consecutive list positions (positions past the end of the group repeat `first`).  The list
 // entries are requested together and without a branch around the loads (a load under a branch is waited for
 // where the branches join: one memory round trip per row); without a list the same loads read the head of
 // the activations, which is always there, and their values are dropped.
-template <int R>
-__device__ __forceinline__ void sgmv_rows(const SgmvArgs& a, int first, int n_left, int (&rows)[R]) {
+template <int R, class T>
+__device__ __forceinline__ void sgmv_rows(const SgmvArgsT<T>& a, int first, int n_left, int (&rows)[R]) {
   const int* list = a.perm ? a.perm : reinterpret_cast<const int*>(a.x);
   int pos[R], listed[R];
 #pragma unroll
@@ -167,12 +176,12 @@ __device__ __forceinline__ void sgmv_rows(const SgmvArgs& a, int first, int n_le
 // wavefront's loads cover consecutive memory; the matching two activations of a row are one dword.
 // Each thread keeps R x 8 partial sums; they are summed over the threads of a column block in two
 // passes through LDS (row stride 8 R + 1 floats, so neither pass has bank conflicts worth naming).
-template <int DOUT, int R>
-__global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgs a) {
+template <int DOUT, int R, class T>
+__global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgsT<T> a) {
   constexpr int V = 8 * R;
   __shared__ float part[256 * (V + 1)];
   __shared__ float part2[256];
-  SgmvGroup g;
+  SgmvGroupT<T> g;
   if (!sgmv_group(a, blockIdx.x, &g)) return;
   const int tid = threadIdx.x;
   const int dn = a.d_out;
@@ -185,8 +194,8 @@ __global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgs a) {
   const int v2 = tid % V, cb2 = (tid / V) % CB, part_id = tid / (V * CB);
   for (int r0 = blockIdx.y * R; r0 < g.count; r0 += gridDim.y * R) {
     int rows[R];
-    const _Float16* xr[R];
-    sgmv_rows<R>(a, g.start + r0, g.count - r0, rows);
+    const T* xr[R];
+    sgmv_rows<R, T>(a, g.start + r0, g.count - r0, rows);
 #pragma unroll
     for (int r = 0; r < R; r++) xr[r] = a.x + (long)rows[r] * a.x_stride;
     float acc[R][8];
@@ -200,19 +209,19 @@ __global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgs a) {
       // has U times the requests in flight and a U-th of the round trips in sequence.  Sums are taken in
       // the order of k, as without the batching.
       constexpr int U = TRITEIA_SHRINK_UNROLL;
-      const _Float16* wp = g.w + cb * 8;
+      const T* wp = g.w + cb * 8;
       const int kstep = 2 * KP;
       for (int k0 = 2 * kp; k0 < a.d_in; k0 += U * kstep) {
-        lhalf8_t w0[U], w1[U];
-        lhalf2_t xv[U][R];
+        lvec8<T> w0[U], w1[U];
+        lvec2<T> xv[U][R];
 #pragma unroll
         for (int u = 0; u < U; u++) {
           const int k = k0 + u * kstep;
           const int kc = k < a.d_in ? k : k0;
-          w0[u] = load_global(reinterpret_cast<const lhalf8_t*>(wp + (long)kc * dn));
-          w1[u] = load_global(reinterpret_cast<const lhalf8_t*>(wp + (long)(kc + 1) * dn));
+          w0[u] = load_global(reinterpret_cast<const lvec8<T>*>(wp + (long)kc * dn));
+          w1[u] = load_global(reinterpret_cast<const lvec8<T>*>(wp + (long)(kc + 1) * dn));
 #pragma unroll
-          for (int r = 0; r < R; r++) xv[u][r] = *reinterpret_cast<const lhalf2_t*>(xr[r] + kc);
+          for (int r = 0; r < R; r++) xv[u][r] = *reinterpret_cast<const lvec2<T>*>(xr[r] + kc);
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
@@ -245,8 +254,8 @@ __global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgs a) {
         int row = rows[0];
 #pragma unroll
         for (int q = 1; q < R; q++) row = r == q ? rows[q] : row;
-        _Float16* yp = a.y + (long)row * a.y_stride + cb2 * 8 + (v2 & 7);
-        *yp = (_Float16)((float)*yp + sum * a.scale);
+        T* yp = a.y + (long)row * a.y_stride + cb2 * 8 + (v2 & 7);
+        *yp = (T)((float)*yp + sum * a.scale);
       }
     }
   }
@@ -254,10 +263,10 @@ __global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgs a) {
 
 // narrow -> wide (d_in <= 128): grid (n_groups, ceil(d_out / 256)), block 256;
 // each thread keeps its weight column in registers and walks the group's rows.
-template <int DIN>
-__global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgs a) {
+template <int DIN, class T>
+__global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgsT<T> a) {
   __shared__ float xs[DIN];
-  SgmvGroup g;
+  SgmvGroupT<T> g;
   if (!sgmv_group(a, blockIdx.x, &g)) return;
   const int j = blockIdx.y * 256 + threadIdx.x;
   const bool ok = j < a.d_out;
@@ -273,8 +282,8 @@ __global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgs a) {
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < DIN; i++) acc += w[i] * xs[i];
-      _Float16* yp = a.y + (long)row * a.y_stride + j;
-      *yp = (_Float16)((float)*yp + acc * a.scale);
+      T* yp = a.y + (long)row * a.y_stride + j;
+      *yp = (T)((float)*yp + acc * a.scale);
     }
   }
 }
@@ -283,9 +292,9 @@ __global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgs a) {
 // A thread owns 8 consecutive output columns: its d_in x 8 weight patch stays in registers while
 // it walks the group's rows R at a time (16-byte loads and stores throughout, no barriers; the R
 // rows' loads are independent, so they are in flight together).
-template <int DIN, int R>
-__global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgs a) {
-  SgmvGroup g;
+template <int DIN, int R, class T>
+__global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgsT<T> a) {
+  SgmvGroupT<T> g;
   if (!sgmv_group(a, blockIdx.x, &g)) return;
   const int j0 = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (j0 >= a.d_out) return;
@@ -294,29 +303,29 @@ __global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgs a) 
   // Order of the requests: the first rows' list entries, then the weight patch, then (once the rows are
   // known) their activations and old outputs; nothing is waited for before all of these are on their way.
   int rows[R];
-  sgmv_rows<R>(a, g.start + r0, g.count - r0, rows);
-  lhalf8_t w[DIN];
+  sgmv_rows<R, T>(a, g.start + r0, g.count - r0, rows);
+  lvec8<T> w[DIN];
 #pragma unroll
   for (int i = 0; i < DIN; i++)   // (no branch around a load: rows past d_in re-read the last one and are zeroed below)
-    w[i] = load_global(reinterpret_cast<const lhalf8_t*>(g.w + (long)(i < a.d_in ? i : a.d_in - 1) * a.d_out + j0));
+    w[i] = load_global(reinterpret_cast<const lvec8<T>*>(g.w + (long)(i < a.d_in ? i : a.d_in - 1) * a.d_out + j0));
   bool patch_ready = false;
   for (;;) {
-    lhalf8_t xv[R][DIN / 8], old[R];
-    _Float16* yp[R];
+    lvec8<T> xv[R][DIN / 8], old[R];
+    T* yp[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      const _Float16* xr = a.x + (long)rows[r] * a.x_stride;
+      const T* xr = a.x + (long)rows[r] * a.x_stride;
       yp[r] = a.y + (long)rows[r] * a.y_stride + j0;
 #pragma unroll
       for (int i0 = 0; i0 < DIN / 8; i0++)
-        xv[r][i0] = *reinterpret_cast<const lhalf8_t*>(xr + (i0 * 8 < a.d_in ? i0 * 8 : 0));   // same address in every lane
-      old[r] = *reinterpret_cast<const lhalf8_t*>(yp[r]);
+        xv[r][i0] = *reinterpret_cast<const lvec8<T>*>(xr + (i0 * 8 < a.d_in ? i0 * 8 : 0));   // same address in every lane
+      old[r] = *reinterpret_cast<const lvec8<T>*>(yp[r]);
     }
     __builtin_amdgcn_sched_barrier(0);   // every request above is issued before the first result is touched
     if (!patch_ready) {
 #pragma unroll
       for (int i = 0; i < DIN; i++)
-        if (i >= a.d_in) w[i] = lhalf8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if (i >= a.d_in) w[i] = lvec8<T>{0, 0, 0, 0, 0, 0, 0, 0};
       patch_ready = true;
     }
     const int n_left = g.count - r0;
@@ -329,14 +338,14 @@ __global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgs a) 
       for (int i = 0; i < DIN; i++)
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] += (float)xv[r][i / 8][i % 8] * (float)w[i][e];
-      lhalf8_t o;
+      lvec8<T> o;
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = (_Float16)((float)old[r][e] + acc[e] * a.scale);
-      if (r == 0 || r < n_left) *reinterpret_cast<lhalf8_t*>(yp[r]) = o;
+      for (int e = 0; e < 8; e++) o[e] = (T)((float)old[r][e] + acc[e] * a.scale);
+      if (r == 0 || r < n_left) *reinterpret_cast<lvec8<T>*>(yp[r]) = o;
     }
     r0 += gridDim.z * R;
     if (r0 >= g.count) break;
-    sgmv_rows<R>(a, g.start + r0, g.count - r0, rows);
+    sgmv_rows<R, T>(a, g.start + r0, g.count - r0, rows);
   }
 }
 

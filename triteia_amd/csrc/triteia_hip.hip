@@ -820,8 +820,14 @@ int triteia_hip_sbmm_2_4_routed_static(const void* A, const void* B, const void*
                                      kStaticPlanBytes, accumulate, -1, stream);
 }
 
-int triteia_hip_bgmv(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
-                     int num_layers, int layer_idx, float scale, int dev, void* stream) {
+}  // extern "C"
+
+namespace {
+typedef __bf16 bf16_t;
+
+template <class T>
+int bgmv_impl(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out, int num_layers,
+              int layer_idx, float scale, int dev, void* stream) {
   if (batch < 0 || h_in <= 0 || h_out <= 0 || num_layers <= 0 || layer_idx < 0 || layer_idx >= num_layers)
     return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "bgmv: batch=%d h_in=%d h_out=%d layers=%d layer=%d", batch, h_in, h_out, num_layers, layer_idx);
   const int narrow = h_in < h_out ? h_in : h_out;
@@ -833,20 +839,15 @@ int triteia_hip_bgmv(void* Y, const void* X, const void* W, const void* indices,
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (h_in >= h_out) {
-    hipLaunchKernelGGL(bgmv_shrink_kernel, dim3(batch), dim3(256), 0, st, static_cast<_Float16*>(Y),
-                       static_cast<const _Float16*>(X), static_cast<const _Float16*>(W),
-                       static_cast<const long long*>(indices), h_in, h_out, (long)num_layers, (long)layer_idx, scale);
+    hipLaunchKernelGGL(bgmv_shrink_kernel<T>, dim3(batch), dim3(256), 0, st, static_cast<T*>(Y), static_cast<const T*>(X),
+                       static_cast<const T*>(W), static_cast<const long long*>(indices), h_in, h_out, (long)num_layers,
+                       (long)layer_idx, scale);
   } else {
-    hipLaunchKernelGGL(bgmv_expand_kernel, dim3((h_out + 255) / 256, batch), dim3(256), 0, st, static_cast<_Float16*>(Y),
-                       static_cast<const _Float16*>(X), static_cast<const _Float16*>(W),
-                       static_cast<const long long*>(indices), h_in, h_out, (long)num_layers, (long)layer_idx, scale);
+    hipLaunchKernelGGL(bgmv_expand_kernel<T>, dim3((h_out + 255) / 256, batch), dim3(256), 0, st, static_cast<T*>(Y),
+                       static_cast<const T*>(X), static_cast<const T*>(W), static_cast<const long long*>(indices), h_in,
+                       h_out, (long)num_layers, (long)layer_idx, scale);
   }
   return check_launch("bgmv kernel");
-}
-
-size_t triteia_hip_sgmv_tmp_size(int num_problems) {
-  // the reference's CUTLASS argument block: 60 bytes per problem (sgmv.cuh:48-52)
-  return num_problems > 0 ? (size_t)60 * (size_t)num_problems : 0;
 }
 
 #ifndef TRITEIA_SHRINK_ROWS16
@@ -858,7 +859,8 @@ size_t triteia_hip_sgmv_tmp_size(int num_problems) {
 constexpr int kShrinkRows16 = TRITEIA_SHRINK_ROWS16;   // token rows a block of the rank <= 16 shrink kernel takes at a time
 constexpr int kExpandRows16 = TRITEIA_EXPAND_ROWS16;
 
-static int launch_sgmv(SgmvArgs a, int max_rows, hipStream_t st) {
+template <class T>
+int launch_sgmv(SgmvArgsT<T> a, int max_rows, hipStream_t st) {
   const int narrow = a.d_in < a.d_out ? a.d_in : a.d_out;
   if (a.d_in % 8 != 0 || a.d_out % 8 != 0 || narrow > kLoraMaxNarrow)
     return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "No suitable kernel. d_in=%d d_out=%d", a.d_in, a.d_out);
@@ -868,36 +870,36 @@ static int launch_sgmv(SgmvArgs a, int max_rows, hipStream_t st) {
   if (row_slots < 1) row_slots = 1;
   auto slots = [&](int rows_per_block) { return (row_slots + rows_per_block - 1) / rows_per_block; };
   if (a.d_in >= a.d_out) {
-    if (a.d_out <= 16) hipLaunchKernelGGL((sgmv_shrink_kernel<16, kShrinkRows16>), dim3(a.n_groups, slots(kShrinkRows16)), dim3(256), 0, st, a);
-    else if (a.d_out <= 32) hipLaunchKernelGGL((sgmv_shrink_kernel<32, 2>), dim3(a.n_groups, slots(2)), dim3(256), 0, st, a);
-    else if (a.d_out <= 64) hipLaunchKernelGGL((sgmv_shrink_kernel<64, 1>), dim3(a.n_groups, slots(1)), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((sgmv_shrink_kernel<128, 1>), dim3(a.n_groups, slots(1)), dim3(256), 0, st, a);
+    if (a.d_out <= 16) hipLaunchKernelGGL((sgmv_shrink_kernel<16, kShrinkRows16, T>), dim3(a.n_groups, slots(kShrinkRows16)), dim3(256), 0, st, a);
+    else if (a.d_out <= 32) hipLaunchKernelGGL((sgmv_shrink_kernel<32, 2, T>), dim3(a.n_groups, slots(2)), dim3(256), 0, st, a);
+    else if (a.d_out <= 64) hipLaunchKernelGGL((sgmv_shrink_kernel<64, 1, T>), dim3(a.n_groups, slots(1)), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((sgmv_shrink_kernel<128, 1, T>), dim3(a.n_groups, slots(1)), dim3(256), 0, st, a);
   } else {
     const int rz = row_slots < 8 ? row_slots : 8;
     const dim3 grid(a.n_groups, (a.d_out + 255) / 256, rz);
     const int col_blocks = (a.d_out + 2047) / 2048;
-    if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_vec_kernel<16, kExpandRows16>), dim3(a.n_groups, col_blocks, slots(kExpandRows16)), dim3(256), 0, st, a);
-    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_vec_kernel<32, 2>), dim3(a.n_groups, col_blocks, slots(2)), dim3(256), 0, st, a);
-    else if (a.d_in <= 64) hipLaunchKernelGGL((sgmv_expand_kernel<64>), grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((sgmv_expand_kernel<128>), grid, dim3(256), 0, st, a);
+    if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_vec_kernel<16, kExpandRows16, T>), dim3(a.n_groups, col_blocks, slots(kExpandRows16)), dim3(256), 0, st, a);
+    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_vec_kernel<32, 2, T>), dim3(a.n_groups, col_blocks, slots(2)), dim3(256), 0, st, a);
+    else if (a.d_in <= 64) hipLaunchKernelGGL((sgmv_expand_kernel<64, T>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((sgmv_expand_kernel<128, T>), grid, dim3(256), 0, st, a);
   }
   return check_launch("sgmv kernel");
 }
 
-int triteia_hip_sgmv(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
-                     int d_out, int layer_idx, int dev, void* stream) {
-  (void)tmp;
+template <class T>
+int sgmv_impl(void* y, const void* x, const void* w_ptrs, const void* s, int num_problems, int d_in, int d_out, int layer_idx,
+              int dev, void* stream) {
   if (num_problems < 0 || d_in <= 0 || d_out <= 0 || layer_idx < 0)
     return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sgmv: problems=%d d_in=%d d_out=%d layer=%d", num_problems, d_in, d_out, layer_idx);
   if (num_problems == 0) return TRITEIA_HIP_OK;
   if (!y || !x || !w_ptrs || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sgmv: null tensor pointer");
   DeviceGuard g(dev);
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
-  SgmvArgs a;
+  SgmvArgsT<T> a;
   memset(&a, 0, sizeof(a));
-  a.y = static_cast<_Float16*>(y);
+  a.y = static_cast<T*>(y);
   a.y_stride = d_out;
-  a.x = static_cast<const _Float16*>(x);
+  a.x = static_cast<const T*>(x);
   a.x_stride = d_in;
   a.d_in = d_in;
   a.d_out = d_out;
@@ -911,9 +913,9 @@ int triteia_hip_sgmv(void* y, const void* x, const void* w_ptrs, const void* s, 
   return launch_sgmv(a, 64, static_cast<hipStream_t>(stream));
 }
 
-int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
-                            int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
-                            int dev, void* stream) {
+template <class T>
+int sgmv_routed_impl(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride, int n_adapters,
+                     int d_in, int d_out, float scale, const void* plan, int prob_n, int dev, void* stream) {
   if (prob_n < 0 || n_adapters < 0 || d_in <= 0 || d_out <= 0)
     return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sgmv_routed: tokens=%d adapters=%d d_in=%d d_out=%d", prob_n, n_adapters, d_in, d_out);
   if (prob_n == 0 || n_adapters == 0) return TRITEIA_HIP_OK;
@@ -922,15 +924,15 @@ int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   const PlanLayout L = plan_layout(prob_n, n_adapters);
   const int* ws = static_cast<const int*>(plan);
-  SgmvArgs a;
+  SgmvArgsT<T> a;
   memset(&a, 0, sizeof(a));
-  a.y = static_cast<_Float16*>(y);
+  a.y = static_cast<T*>(y);
   a.y_stride = y_stride;
-  a.x = static_cast<const _Float16*>(x);
+  a.x = static_cast<const T*>(x);
   a.x_stride = x_stride;
   a.d_in = d_in;
   a.d_out = d_out;
-  a.w_base = static_cast<const _Float16*>(w_base);
+  a.w_base = static_cast<const T*>(w_base);
   a.w_stride = w_stride;
   // a plan with wide tiles also lists all its tokens in narrow tiles: that is the cut for LoRA
   const bool wide = plan_has_wide(prob_n, n_adapters);
@@ -941,6 +943,45 @@ int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride
   a.n_adapters = n_adapters;
   a.scale = scale;
   return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+extern "C" {
+
+int triteia_hip_bgmv(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                     int num_layers, int layer_idx, float scale, int dev, void* stream) {
+  return bgmv_impl<_Float16>(Y, X, W, indices, batch, h_in, h_out, num_layers, layer_idx, scale, dev, stream);
+}
+int triteia_hip_bgmv_bf16(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                          int num_layers, int layer_idx, float scale, int dev, void* stream) {
+  return bgmv_impl<bf16_t>(Y, X, W, indices, batch, h_in, h_out, num_layers, layer_idx, scale, dev, stream);
+}
+
+size_t triteia_hip_sgmv_tmp_size(int num_problems) {
+  // the reference's CUTLASS argument block: 60 bytes per problem (sgmv.cuh:48-52)
+  return num_problems > 0 ? (size_t)60 * (size_t)num_problems : 0;
+}
+
+int triteia_hip_sgmv(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
+                     int d_out, int layer_idx, int dev, void* stream) {
+  (void)tmp;
+  return sgmv_impl<_Float16>(y, x, w_ptrs, s, num_problems, d_in, d_out, layer_idx, dev, stream);
+}
+int triteia_hip_sgmv_bf16(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
+                          int d_out, int layer_idx, int dev, void* stream) {
+  (void)tmp;
+  return sgmv_impl<bf16_t>(y, x, w_ptrs, s, num_problems, d_in, d_out, layer_idx, dev, stream);
+}
+
+int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
+                            int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
+                            int dev, void* stream) {
+  return sgmv_routed_impl<_Float16>(y, y_stride, x, x_stride, w_base, w_stride, n_adapters, d_in, d_out, scale, plan, prob_n, dev, stream);
+}
+int triteia_hip_sgmv_routed_bf16(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
+                                 int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
+                                 int dev, void* stream) {
+  return sgmv_routed_impl<bf16_t>(y, y_stride, x, x_stride, w_base, w_stride, n_adapters, d_in, d_out, scale, plan, prob_n, dev, stream);
 }
 
 }  // extern "C"

@@ -43,6 +43,10 @@ SIGNATURES = {
     "triteia_hip_bgmv": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_float, _c_int, _c_vp]),
     "triteia_hip_sgmv": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp]),
     "triteia_hip_sgmv_tmp_size": (_c_sz, [_c_int]),
+    "triteia_hip_bgmv_bf16": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_float, _c_int, _c_vp]),
+    "triteia_hip_sgmv_bf16": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp]),
+    "triteia_hip_sgmv_routed_bf16": (_c_int, [_c_vp, _c_long, _c_vp, _c_long, _c_vp, _c_long] + [_c_int] * 3
+                                     + [_c_float, _c_vp, _c_int, _c_int, _c_vp]),
     "triteia_hip_sgmv_routed": (_c_int, [_c_vp, _c_long, _c_vp, _c_long, _c_vp, _c_long] + [_c_int] * 3
                                 + [_c_float, _c_vp, _c_int, _c_int, _c_vp]),
 }

@@ -4,6 +4,19 @@ import torch
 from . import _ffi
 
 
+_LORA_DTYPES = (torch.float16, torch.bfloat16)
+
+
+def _lora_dtype(x, **others):
+    """fp16 or bf16, the same for every tensor of the call (the reference dispatches on x's dtype and
+    checks the others against it: ops.cpp:132-143, 199-214)."""
+    if x.dtype not in _LORA_DTYPES:
+        raise RuntimeError(f"x must be torch.float16 or torch.bfloat16, got {x.dtype}")
+    for name, t in others.items():
+        _ffi.require_dtype(t, x.dtype, name)
+    return x.dtype
+
+
 def _check(err):
     if err == _ffi.ERR_KERN_SHAPE:
         raise RuntimeError(_ffi.last_error())
@@ -17,8 +30,7 @@ def sgmv(y, x, w_ptr, s, tmp, layer_idx):
     _ffi.require_gpu(y=y, x=x, w_ptr=w_ptr, s=s, tmp=tmp)
     if y.dim() != 2 or x.dim() != 2 or w_ptr.dim() != 1 or s.dim() != 1 or tmp.dim() != 1:
         raise RuntimeError("y, x must be 2D tensors; w_ptr, s, tmp 1D tensors")
-    _ffi.require_dtype(x, torch.float16, "x")
-    _ffi.require_dtype(y, torch.float16, "y")
+    dtype = _lora_dtype(x, y=y)
     _ffi.require_dtype(w_ptr, torch.int64, "w_ptr")
     _ffi.require_dtype(s, torch.int32, "s")
     num_problems = s.size(0) - 1
@@ -27,7 +39,8 @@ def sgmv(y, x, w_ptr, s, tmp, layer_idx):
     if tmp.numel() * tmp.element_size() != sgmv_tmp_size(num_problems):
         raise RuntimeError(f"CHECK_EQ(tmp.size(0), sgmv_tmp_size(num_problems)) failed. "
                            f"{tmp.numel()} vs {sgmv_tmp_size(num_problems)}")
-    _check(_ffi.lib().triteia_hip_sgmv(
+    fn = _ffi.lib().triteia_hip_sgmv if dtype == torch.float16 else _ffi.lib().triteia_hip_sgmv_bf16
+    _check(fn(
         _ffi.ptr(y), _ffi.ptr(x), _ffi.ptr(w_ptr), _ffi.ptr(s), _ffi.ptr(tmp), num_problems, x.size(1), y.size(1),
         int(layer_idx), _ffi.device_index(x), _ffi.stream_of(x)))
 
@@ -41,9 +54,7 @@ def dispatch_bgmv(y, x, w, indicies, layer_idx, scale):
     _ffi.require_gpu(y=y, x=x, w=w, indicies=indicies)
     if y.dim() != 2 or x.dim() != 2 or w.dim() != 4 or indicies.dim() != 1:
         raise RuntimeError("y, x must be 2D tensors, w a 4D tensor, indicies a 1D tensor")
-    _ffi.require_dtype(x, torch.float16, "x")
-    _ffi.require_dtype(y, torch.float16, "y")
-    _ffi.require_dtype(w, torch.float16, "w")
+    dtype = _lora_dtype(x, y=y, w=w)
     _ffi.require_dtype(indicies, torch.int64, "indicies")
     B, h_in = x.shape
     h_out = y.size(1)
@@ -51,7 +62,8 @@ def dispatch_bgmv(y, x, w, indicies, layer_idx, scale):
                        (indicies.size(0), B, "indicies.size(0), x.size(0)"), (y.size(0), B, "y.size(0), x.size(0)")):
         if a != b:
             raise RuntimeError(f"CHECK_EQ({what}) failed. {a} vs {b}")
-    _check(_ffi.lib().triteia_hip_bgmv(
+    fn = _ffi.lib().triteia_hip_bgmv if dtype == torch.float16 else _ffi.lib().triteia_hip_bgmv_bf16
+    _check(fn(
         _ffi.ptr(y), _ffi.ptr(x), _ffi.ptr(w), _ffi.ptr(indicies), B, h_in, h_out, w.size(1), int(layer_idx),
         float(scale), _ffi.device_index(x), _ffi.stream_of(x)))
 
@@ -82,15 +94,14 @@ def add_lora_bgmv(y, x, wa_T_all, wb_T_all, indicies, layer_idx, scale):
 def sgmv_routed(y, x, weights, plan, scale=1.0):
     """y[t] += scale * x[t] @ weights[a] for every token t the routing plan lists under adapter a.
 
-    weights [n_adapters, d_in, d_out] fp16 contiguous; `plan` from capi.route_plan with
+    weights [n_adapters, d_in, d_out] fp16 or bf16 (as x and y), contiguous; `plan` from capi.route_plan with
     n_deltas == n_adapters."""
     _ffi.require_gpu(y=y, x=x, weights=weights, plan=plan)
-    _ffi.require_dtype(x, torch.float16, "x")
-    _ffi.require_dtype(y, torch.float16, "y")
-    _ffi.require_dtype(weights, torch.float16, "weights")
+    dtype = _lora_dtype(x, y=y, weights=weights)
     n_adapters, d_in, d_out = weights.shape
     if x.size(1) != d_in or y.size(1) != d_out or x.size(0) != y.size(0):
         raise RuntimeError("shape mismatch between x, y and weights")
-    _check(_ffi.lib().triteia_hip_sgmv_routed(
+    fn = _ffi.lib().triteia_hip_sgmv_routed if dtype == torch.float16 else _ffi.lib().triteia_hip_sgmv_routed_bf16
+    _check(fn(
         _ffi.ptr(y), y.stride(0), _ffi.ptr(x), x.stride(0), _ffi.ptr(weights), d_in * d_out, n_adapters, d_in, d_out,
         float(scale), _ffi.ptr(plan), x.size(0), _ffi.device_index(x), _ffi.stream_of(x)))
