@@ -379,6 +379,66 @@ def run_sweep(torch, ffi):
     return out
 
 
+def measure_lora(torch, ffi, tokens=256, adapters=32, k=4096, m=11008, rank=16, calls=20):
+    """The LoRA companions at configuration 3's shape (rank-16 adapters on 4096 x 11008, the routing of cfg3): BGMV
+    (one adapter look-up per token) and routed SGMV (tokens grouped by a routing plan), each as shrink + expand, timed
+    as `calls` pairs in one captured HIP graph.  Bytes: every distinct adapter once, activations, the rank-r
+    intermediate written and read, the output read and written."""
+    from triteia_amd import workloads as W
+    from triteia_amd.python.capi import add_lora_bgmv, route_plan, sgmv_routed
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(77)
+    x = W.random_activations(tokens, k, 78, dev)
+    A = (torch.randn((adapters, k, rank), generator=g, device=dev) * 0.01).half()
+    B = (torch.randn((adapters, rank, m), generator=g, device=dev) * 0.01).half()
+    A_t = A.transpose(1, 2).contiguous().unsqueeze(1)      # BGMV's layout: [n, layers, out, in]
+    B_t = B.transpose(1, 2).contiguous().unsqueeze(1)
+    idx_np = W.zipf_indices(tokens, adapters, 1.5, 1003, 0.10)
+    idx32 = torch.from_numpy(idx_np).to(dev)
+    idx64 = idx32.to(torch.long)
+    y = torch.zeros((tokens, m), dtype=torch.float16, device=dev)
+    v = torch.zeros((tokens, rank), dtype=torch.float16, device=dev)
+    plan = route_plan(idx32, adapters)
+    used = len(set(int(i) for i in idx_np if i >= 0))
+    routed = int((idx_np >= 0).sum())
+    nbytes = used * (k * rank + rank * m) * 2 + routed * (k * 2 + 4 * rank + 4 * m)
+
+    def bgmv():
+        add_lora_bgmv(y, x, A_t, B_t, idx64, 0, 1.0)
+
+    def sgmv():
+        v.zero_()
+        sgmv_routed(v, x, A, plan)
+        sgmv_routed(y, v, B, plan)
+
+    out = []
+    for name, fn, kernels in (("lora_bgmv", bgmv, "bgmv_shrink_kernel + bgmv_expand_kernel"),
+                              ("lora_sgmv_routed", sgmv, "sgmv_shrink_kernel + sgmv_expand_vec_kernel")):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(calls):
+                    fn()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        us = (time.perf_counter() - t0) / calls * 1e6
+        del graph
+        out.append({"workload": f"{name} rank {rank}, {adapters} adapters on {k}x{m}, {tokens} tokens Zipf(1.5)", "tokens": tokens,
+                    "tokens_routed": routed, "deltas_used": used, "ms_per_step": round(us * 1e-3, 5),
+                    "tflops": round(2.0 * routed * rank * (k + m) / (us * 1e-6) / 1e12, 2), "kernel": kernels,
+                    "kernel_us": round(us, 2), "bound": "hbm", "frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+    return out
+
+
 def host_call_us(prob, wl, torch, n=300):
     """Host time of one `ops.sbmm_4bit_2_4_native` call (Python mirror -> ctypes -> C ABI), launches left to queue up."""
     if wl.op != "sbmm":
@@ -490,7 +550,7 @@ def main():
     del prob
     torch.cuda.empty_cache()
     if not a.no_sweep and a.workload == "cfg2" and a.tokens is None:
-        res["sweep"] = run_sweep(torch, ffi)
+        res["sweep"] = run_sweep(torch, ffi) + measure_lora(torch, ffi)
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl, torch)
     print(json.dumps(res))

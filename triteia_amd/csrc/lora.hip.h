@@ -42,55 +42,146 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // ---------------------------------------------------------------- BGMV ----
 
-// wide -> narrow: grid (B), block 256.  Wave w computes outputs j = w, w+4, ...
+// wide -> narrow: grid (B), block 256.  The block walks the token's activations once per 16 outputs: thread t takes the
+// 8-element pieces t, t + 256, ... of x and of each of the 16 weight rows (all of a piece's loads are independent, so
+// they are in flight together), then the 16 partial sums are added over the wavefront by shuffles and over the four
+// wavefronts through LDS.
 template <class T>
 __global__ __launch_bounds__(256) void bgmv_shrink_kernel(T* __restrict__ Y, const T* __restrict__ X,
                                                          const T* __restrict__ W,
                                                          const long long* __restrict__ indices, int h_in, int h_out,
                                                          long num_layers, long layer_idx, float scale) {
+  __shared__ float red[4][16];
   const int b = blockIdx.x;
   const long idx = indices[b];
   if (idx < 0) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* w = W + (idx * num_layers + layer_idx) * (long)h_out * h_in;
   const T* x = X + (long)b * h_in;
-  for (int j = wave; j < h_out; j += 4) {
-    const T* wj = w + (long)j * h_in;
-    float acc = 0.f;
-    for (int i = lane * 8; i < h_in; i += 512) {
-      const lvec8<T> wv = *reinterpret_cast<const lvec8<T>*>(wj + i);
-      const lvec8<T> xv = *reinterpret_cast<const lvec8<T>*>(x + i);
+  for (int oc = 0; oc < h_out; oc += 16) {
+    const int n_out = h_out - oc < 16 ? h_out - oc : 16;      // 16, or 8 for the last chunk (h_out is a multiple of 8)
+    float acc[16];
 #pragma unroll
-      for (int e = 0; e < 8; e++) acc += (float)wv[e] * (float)xv[e];
+    for (int j = 0; j < 16; j++) acc[j] = 0.f;
+    for (int i = threadIdx.x * 8; i < h_in; i += 2048) {
+      const lvec8<T> xv = *reinterpret_cast<const lvec8<T>*>(x + i);
+      lvec8<T> wv[16];
+#pragma unroll
+      for (int j = 0; j < 16; j++)   // (rows past the chunk re-read its first row: no branch around a load)
+        wv[j] = *reinterpret_cast<const lvec8<T>*>(w + (long)(oc + (j < n_out ? j : 0)) * h_in + i);
+#pragma unroll
+      for (int j = 0; j < 16; j++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[j] += (float)wv[j][e] * (float)xv[e];
     }
-    acc = wave_sum(acc) * scale;
-    if (lane == 0) Y[(long)b * h_out + j] = (T)((float)Y[(long)b * h_out + j] + acc);
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+      const float sum = wave_sum(acc[j]);
+      if (lane == 0) red[wave][j] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x < n_out) {
+      const float sum = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+      T* yp = Y + (long)b * h_out + oc + threadIdx.x;
+      *yp = (T)((float)*yp + sum * scale);
+    }
+    __syncthreads();
   }
 }
 
-// narrow -> wide: grid (ceil(h_out / 256), B), block 256, one output per thread
+// narrow -> wide: grid (ceil(h_out / 2048), B), block 256.  A thread owns 8 consecutive outputs: their 8 weight rows are
+// one contiguous piece of memory (h_in elements each), the token's h_in activations are the same address in every lane,
+// and the old outputs are one 16-byte load; everything is requested before the first result is used.
 template <class T>
 __global__ __launch_bounds__(256) void bgmv_expand_kernel(T* __restrict__ Y, const T* __restrict__ X,
                                                          const T* __restrict__ W,
                                                          const long long* __restrict__ indices, int h_in, int h_out,
                                                          long num_layers, long layer_idx, float scale) {
-  __shared__ float xs[kLoraMaxNarrow];
   const int b = blockIdx.y;
   const long idx = indices[b];
   if (idx < 0) return;
-  if (threadIdx.x < h_in) xs[threadIdx.x] = (float)X[(long)b * h_in + threadIdx.x];
-  __syncthreads();
-  const int j = blockIdx.x * 256 + threadIdx.x;
-  if (j >= h_out) return;
-  const T* wj = W + ((idx * num_layers + layer_idx) * (long)h_out + j) * h_in;
-  float acc = 0.f;
-  for (int i = 0; i < h_in; i += 8) {
-    const lvec8<T> wv = *reinterpret_cast<const lvec8<T>*>(wj + i);
+  const int j0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (j0 >= h_out) return;
+  const T* w = W + ((idx * num_layers + layer_idx) * (long)h_out + j0) * h_in;
+  const T* x = X + (long)b * h_in;
+  T* yp = Y + (long)b * h_out + j0;
+  const lvec8<T> old = *reinterpret_cast<const lvec8<T>*>(yp);
+  float acc[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) acc += (float)wv[e] * xs[i + e];
+  for (int e = 0; e < 8; e++) acc[e] = 0.f;
+  for (int i = 0; i < h_in; i += 8) {
+    const lvec8<T> xv = *reinterpret_cast<const lvec8<T>*>(x + i);
+    lvec8<T> wv[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) wv[e] = *reinterpret_cast<const lvec8<T>*>(w + (long)e * h_in + i);
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+#pragma unroll
+      for (int q = 0; q < 8; q++) acc[e] += (float)wv[e][q] * (float)xv[q];
   }
-  T* yp = Y + (long)b * h_out + j;
-  *yp = (T)((float)*yp + acc * scale);
+  lvec8<T> o;
+#pragma unroll
+  for (int e = 0; e < 8; e++) o[e] = (T)((float)old[e] + acc[e] * scale);
+  *reinterpret_cast<lvec8<T>*>(yp) = o;
+}
+
+// The same for h_in = 8 LPR with LPR a power of two (h_in = 8 .. 128), written around whole cache lines: a weight row
+// (h_in elements) is spread over LPR neighbouring lanes, 8 elements each, so that one load instruction of a wavefront
+// covers 1 KB of consecutive memory (64 / LPR rows); with a thread per 8 rows, as above, every load instruction touches
+// 64 different lines for 16 bytes each, and the address unit, not memory, bounds the kernel (measured at rank 16:
+// 18.5 us for 256 tokens on 11008 outputs).  The LPR partial dot products of a row are added by shuffles; lane 0 of the row
+// updates the output.  A block takes TB consecutive tokens; the weights stay in registers from one token to the next
+// and are fetched again only when the adapter changes (sorted batches, the hot adapter of a skewed one).
+// grid (ceil(h_out / (4 Q 64 / LPR)), ceil(B / TB)), block 256.
+template <class T, int LPR, int Q, int TB>
+__global__ __launch_bounds__(256) void bgmv_expand_lines_kernel(T* __restrict__ Y, const T* __restrict__ X,
+                                                               const T* __restrict__ W,
+                                                               const long long* __restrict__ indices, int batch, int h_out,
+                                                               long num_layers, long layer_idx, float scale) {
+  constexpr int h_in = 8 * LPR;
+  constexpr int RPL = 64 / LPR;                      // rows per load instruction of a wavefront
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int sub = lane % LPR, rl = lane / LPR;
+  const int row0 = (blockIdx.x * 4 + wave) * Q * RPL + rl;
+  if ((blockIdx.x * 4 + wave) * Q * RPL >= h_out) return;      // (wave-uniform)
+  const int b0 = blockIdx.y * TB;
+  long idx[TB];
+#pragma unroll
+  for (int t = 0; t < TB; t++) idx[t] = indices[b0 + t < batch ? b0 + t : batch - 1];
+  lvec8<T> wv[Q];
+  long have = -1;
+#pragma unroll
+  for (int t = 0; t < TB; t++) {
+    const int b = b0 + t;
+    if (b >= batch || idx[t] < 0) continue;          // (uniform over the block)
+    const lvec8<T> xv = *reinterpret_cast<const lvec8<T>*>(X + (long)b * h_in + sub * 8);
+    T* yrow = Y + (long)b * h_out;
+    T old[Q];
+#pragma unroll
+    for (int q = 0; q < Q; q++) {                     // (rows past the end re-read the last row; their sums are dropped)
+      const int row = row0 + q * RPL < h_out ? row0 + q * RPL : h_out - 1;
+      old[q] = yrow[row];
+    }
+    if (idx[t] != have) {
+      const T* w = W + (idx[t] * num_layers + layer_idx) * (long)h_out * h_in + sub * 8;
+#pragma unroll
+      for (int q = 0; q < Q; q++) {
+        const int row = row0 + q * RPL < h_out ? row0 + q * RPL : h_out - 1;
+        wv[q] = *reinterpret_cast<const lvec8<T>*>(w + (long)row * h_in);
+      }
+      have = idx[t];
+    }
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+      float acc = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc += (float)wv[q][e] * (float)xv[e];
+#pragma unroll
+      for (int off = 1; off < LPR; off <<= 1) acc += __shfl_xor(acc, off, 64);
+      const int row = row0 + q * RPL;
+      if (sub == 0 && row < h_out) yrow[row] = (T)((float)old[q] + acc * scale);
+    }
+  }
 }
 
 // ---------------------------------------------------------------- SGMV ----

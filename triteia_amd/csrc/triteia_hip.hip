@@ -842,8 +842,19 @@ int bgmv_impl(void* Y, const void* X, const void* W, const void* indices, int ba
     hipLaunchKernelGGL(bgmv_shrink_kernel<T>, dim3(batch), dim3(256), 0, st, static_cast<T*>(Y), static_cast<const T*>(X),
                        static_cast<const T*>(W), static_cast<const long long*>(indices), h_in, h_out, (long)num_layers,
                        (long)layer_idx, scale);
+  } else if (h_in == 8 || h_in == 16 || h_in == 32 || h_in == 64 || h_in == 128) {
+    // weight rows spread over neighbouring lanes (whole cache lines per load instruction), four tokens per block
+    constexpr int Q = 8, TB = 4;
+    const int rows_per_block = 4 * Q * 64 / (h_in / 8);
+    const dim3 grid((h_out + rows_per_block - 1) / rows_per_block, (batch + TB - 1) / TB);
+#define BGMV_LINES(LPR_) hipLaunchKernelGGL((bgmv_expand_lines_kernel<T, LPR_, Q, TB>), grid, dim3(256), 0, st, static_cast<T*>(Y), \
+      static_cast<const T*>(X), static_cast<const T*>(W), static_cast<const long long*>(indices), batch, h_out, (long)num_layers, \
+      (long)layer_idx, scale)
+    if (h_in == 8) BGMV_LINES(1); else if (h_in == 16) BGMV_LINES(2); else if (h_in == 32) BGMV_LINES(4);
+    else if (h_in == 64) BGMV_LINES(8); else BGMV_LINES(16);
+#undef BGMV_LINES
   } else {
-    hipLaunchKernelGGL(bgmv_expand_kernel<T>, dim3((h_out + 255) / 256, batch), dim3(256), 0, st, static_cast<T*>(Y),
+    hipLaunchKernelGGL(bgmv_expand_kernel<T>, dim3((h_out + 2047) / 2048, batch), dim3(256), 0, st, static_cast<T*>(Y),
                        static_cast<const T*>(X), static_cast<const T*>(W), static_cast<const long long*>(indices), h_in,
                        h_out, (long)num_layers, (long)layer_idx, scale);
   }
