@@ -48,6 +48,9 @@ def parse():
     p.add_argument("--no-graph", action="store_true", help="time eager launches instead of one captured HIP graph")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-sweep", action="store_true", help="skip the tokens x deltas sweep (the `sweep` array)")
+    p.add_argument("--probe", action="store_true",
+                   help="measure the two ceilings instead: the headline kernel with its MFMAs left out (what memory alone allows for "
+                        "its access pattern) and loops of sparse MFMAs on random operands (what the matrix cores allow)")
     p.add_argument("--warm-cache", action="store_true", help="do not rotate weight copies (Infinity-Cache-warm number)")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run one plain 256 MiB device copy (a known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -439,6 +442,60 @@ def measure_lora(torch, ffi, tokens=256, adapters=32, k=4096, m=11008, rank=16, 
     return out
 
 
+def run_probes(torch, ffi):
+    """The ceilings the product kernels are priced against, measured on this GPU (one JSON line)."""
+    from triteia_amd import workloads as W
+    lib, P = ffi.lib(), ffi.ptr
+    wl = W.config("cfg2")
+    prob = Problem(wl, copies_for(wl), torch, ffi)
+    torch.cuda.synchronize()
+
+    def timed(call, batch=10, reps=15):
+        for i in range(5):
+            call(i)
+        torch.cuda.synchronize()
+        durs = []
+        for r in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(batch):
+                call(r * batch + i)
+            e1.record()
+            e1.synchronize()
+            durs.append(e0.elapsed_time(e1) / batch * 1e-3)
+        return float(np.median(durs))
+
+    def loads_only(i):
+        q, me, s = prob.weights[i % prob.copies]
+        prob._chk(lib.triteia_hip_probe_stream(P(prob.x), P(q), P(me), P(prob.out), P(s), P(prob.idx), wl.n_deltas, wl.m, wl.tokens,
+                                               wl.k, 0, prob.stream()))
+
+    t_loads, t_real = timed(loads_only), timed(prob.step)
+    nbytes = wl.delta_algorithmic_bytes()
+    out = {"probe": "ceilings", "workload": wl.name, "algorithmic_bytes": nbytes,
+           "stream": {"kernel": "sparse24_grouped_kernel<1, 4, 1, eager> without its MFMAs", "us": round(t_loads * 1e6, 2),
+                      "gbs": round(nbytes / t_loads / 1e9, 1), "frac_of_8_tbs": round(nbytes / t_loads / 1e9 / HBM_PEAK_GBS, 4)},
+           "product_kernel": {"us": round(t_real * 1e6, 2), "gbs": round(nbytes / t_real / 1e9, 1),
+                              "frac_of_8_tbs": round(nbytes / t_real / 1e9 / HBM_PEAK_GBS, 4), "frac_of_stream_probe": round(t_loads / t_real, 4)}}
+    del prob
+    torch.cuda.empty_cache()
+    src = torch.randn(16384, device="cuda:0").half()
+    sink = torch.empty(256 * 512, dtype=torch.float32, device="cuda:0")
+    iters = 4000
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    names = ("32 sparse MFMAs per round, nothing else", "+ 16 LDS reads of 16 bytes per round", "+ 16 LDS reads and 32 conversion pairs per round")
+    out["mfma"] = []
+    for variant, name in enumerate(names):
+        def call(_i, variant=variant):
+            rc = lib.triteia_hip_probe_mfma(variant, iters, P(sink), P(src), 0, stream)
+            assert rc == 0, ffi.last_error()
+        t = timed(call, batch=1, reps=7)
+        flops = 2.0 * 16 * 16 * 64 * 32 * 8 * 256 * iters
+        out["mfma"].append({"loop": name, "ms": round(t * 1e3, 3), "pflops_dense_equivalent": round(flops / t / 1e15, 3),
+                            "frac_of_5_pflops": round(flops / t / 1e15 / 5.0, 4)})
+    print(json.dumps(out))
+
+
 def host_call_us(prob, wl, torch, n=300):
     """Host time of one `ops.sbmm_4bit_2_4_native` call (Python mirror -> ctypes -> C ABI), launches left to queue up."""
     if wl.op != "sbmm":
@@ -469,6 +526,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     ffi.lib()   # fails loudly if the HIP library is missing
+    if a.probe:
+        run_probes(torch, ffi)
+        return
 
     shape = tuple(int(v) for v in a.shape.split(",")) if a.shape else None
     if shape is not None and (a.workload != "cfg0" or len(shape) != 2 or shape[0] % 64 or shape[1] % 128):

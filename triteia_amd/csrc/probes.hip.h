@@ -1,0 +1,58 @@
+// Measurement kernels: what the hardware allows on its own, for pricing the product kernels against.
+// Reached only through the triteia_hip_probe_* entry points (bench.py --probe).
+#pragma once
+#include "sparse24_gemm.hip.h"
+
+namespace triteia_hip {
+
+// Nothing but independent sparse MFMAs on random operands: 256 x 8 wavefronts (two per SIMD), each issuing `iters`
+// rounds of 32 v_smfmac_f32_16x16x64_f16 on 32 accumulators.  `lds_reads` / `valu_pairs` add that many 16-byte LDS
+// reads and (bitfield insert, packed add) pairs per round, the operand traffic and conversion work that a real
+// kernel cannot avoid.  `src`: at least 16 KB of random fp16 values.
+template <int LDS_READS, int VALU_PAIRS>
+__global__ __launch_bounds__(512, 1) void mfma_probe_kernel(int iters, float* out, const _Float16* src) {
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[32768];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < 8192; i += blockDim.x) reinterpret_cast<uint32_t*>(lds)[i] = i * 2654435761u;
+  __syncthreads();
+  float4_t acc[32];
+#pragma unroll
+  for (int i = 0; i < 32; i++) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+  half8_t A[2];
+  half16_t B[4];
+#pragma unroll
+  for (int i = 0; i < 2; i++) A[i] = *reinterpret_cast<const half8_t*>(src + (lane + 64 * i) * 8);
+#pragma unroll
+  for (int i = 0; i < 4; i++) B[i] = *reinterpret_cast<const half16_t*>(src + 1024 + (lane + 64 * i) * 16);
+  const uint32_t base = (uint32_t)(uintptr_t)lds + wave * 4096 + lane * 16;
+  uint32_t w = lane * 77;
+  const int idx = 0x4444;
+  for (int it = 0; it < iters; it++) {
+    uint4_t v[LDS_READS > 0 ? LDS_READS : 1];
+#pragma unroll
+    for (int j = 0; j < LDS_READS; j++) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v[j]) : "v"(base), "n"(j * 1024 % 4096));
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        acc[c * 4 + nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A[c & 1], B[nt], acc[c * 4 + nt], idx, 0, 0);
+#pragma unroll
+      for (int j = 0; j < VALU_PAIRS / 8; j++) {
+        uint32_t t;
+        asm volatile("v_bfi_b32 %0, %1, %2, %3" : "=v"(t) : "s"(0x000f000fu), "v"(w), "v"(0x64006400u));
+        asm volatile("v_pk_add_f16 %0, %1, %2" : "=v"(w) : "v"(t), "v"(w));
+      }
+    }
+    if (LDS_READS > 0) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < LDS_READS; j++) w += v[j][0];
+    }
+  }
+  float s = (float)w;
+#pragma unroll
+  for (int i = 0; i < 32; i++) s += acc[i][0];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+}  // namespace triteia_hip

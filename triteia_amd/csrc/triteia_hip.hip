@@ -11,6 +11,7 @@
 #include <mutex>
 
 #include "lora.hip.h"
+#include "probes.hip.h"
 #include "route_plan.hip.h"
 #include "sparse24_gemm.hip.h"
 #include "sparse24_tile256.hip.h"
@@ -646,6 +647,43 @@ static int plan_has_wide(int prob_n, int n_deltas) {
 int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
   return mid_tiles(prob_n, n_deltas, prob_m, prob_k) ? triteia_hip_plan_tile_tokens(prob_n, n_deltas) : 0;
+}
+
+int triteia_hip_probe_mfma(int variant, int iters, void* out, const void* random_fp16, int dev, void* stream) {
+  if (iters <= 0 || !out || !random_fp16) return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_mfma: iters=%d or a null buffer", iters);
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* o = static_cast<float*>(out);
+  const _Float16* src = static_cast<const _Float16*>(random_fp16);
+  if (variant == 0) hipLaunchKernelGGL((mfma_probe_kernel<0, 0>), dim3(256), dim3(512), 0, st, iters, o, src);
+  else if (variant == 1) hipLaunchKernelGGL((mfma_probe_kernel<16, 0>), dim3(256), dim3(512), 0, st, iters, o, src);
+  else if (variant == 2) hipLaunchKernelGGL((mfma_probe_kernel<16, 32>), dim3(256), dim3(512), 0, st, iters, o, src);
+  else return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_mfma: variant %d", variant);
+  return check_launch("mfma_probe_kernel");
+}
+
+int triteia_hip_probe_stream(const void* A, const void* B, const void* meta, void* C, const void* s, const void* token_indices,
+                             int n_deltas, int prob_m, int prob_n, int prob_k, int dev, void* stream) {
+  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, -1)) return e;
+  if (prob_n <= 0 || prob_n > 64 || n_deltas <= 0 || n_deltas > 16 || !A || !B || !meta || !C || !s || !token_indices)
+    return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_stream: at most 64 tokens over at most 16 deltas, no null pointers");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  // the launch of triteia_hip_sbmm_2_4_routed for such a batch (in-kernel routing, weights requested ahead of it)
+  Sparse24Args a;
+  fill_weights(a, A, B, meta, C, s, prob_m, prob_k, n_deltas);
+  a.raw_indices = static_cast<const int*>(token_indices);
+  a.raw_count = prob_n;
+  a.n_groups = n_deltas;
+  a.raw_static = 1;
+  const long cb_pad = (a.m / 128 + 7) / 8 * 8;
+  const long side_by_side = 512 / cb_pad;
+  const int n_steps = (a.k / 32 + 3) / 4;
+  a.rot_spread = side_by_side >= 4 ? (int)(n_steps / (side_by_side < 16 ? side_by_side : 16)) : 0;
+  hipLaunchKernelGGL((sparse24_grouped_kernel<1, 4, 1, true, true>), dim3((unsigned)(n_deltas * cb_pad)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), a);
+  return check_launch("sparse24_grouped_kernel (loads only)");
 }
 
 int triteia_hip_routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
