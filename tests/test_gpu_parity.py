@@ -149,6 +149,33 @@ def test_split_k_across_workgroups(ops, monkeypatch, b, n, k, m, ks, seed):
     assert float((first.float() - unsplit.float()).norm() / unsplit.float().norm()) < 1e-4
 
 
+@pytest.mark.parametrize("b,n,k,m,seed", [(1, 16, 512, 384, 71), (1, 5, 4096, 256, 72), (3, 1, 1024, 128, 73), (2, 16, 192, 1152, 74)])
+def test_column_shares_keep_the_bits(ops, monkeypatch, b, n, k, m, seed):
+    """Small matmul / bmm launches give a workgroup a share of a column block (64, 32 or 16 columns instead of 128).  Every
+    output column is still summed by the same wavefronts in the same order: each share width gives the bits of the whole block,
+    and the oracle's values."""
+    say(f"column shares b={b} n={n} k={k} m={m} seed={seed}")
+    qw, meta, s = make_deltas(b, k, m, seed)
+    x = activations(b * n, k, seed + 1).reshape(b, n, k)
+    gq, gm, gs, gx = to_gpu(qw, meta, s, x)
+    if b == 1:
+        ref = orc.matmul_4bit_2_4(qw[0], x[0], meta[0], s[0])
+        call = lambda: ops.matmul_4bit_2_4(gq[0], gx[0], gm[0], gs[0])
+    else:
+        ref = orc.bmm_4bit_2_4(qw, x, meta, s)
+        call = lambda: ops.bmm_4bit_2_4(gq, gx, gm, gs)
+    setknob(monkeypatch, "TRITEIA_HIP_KSPLIT", 0)
+    setknob(monkeypatch, "TRITEIA_HIP_SUB_SHIFT", 0)
+    whole = call()
+    torch.cuda.synchronize()
+    check_close(whole, ref, what="whole column blocks")
+    for shift in (1, 2, 3):
+        setknob(monkeypatch, "TRITEIA_HIP_SUB_SHIFT", shift)
+        assert torch.equal(call(), whole), f"shares of {128 >> shift} columns changed the result"
+    delknob(monkeypatch, "TRITEIA_HIP_SUB_SHIFT")
+    assert torch.equal(call(), whole), "the rule's own choice of share changed the result"
+
+
 def test_reference_shaped_entry_points_directly(ops):
     """triteia_hip_mul_2_4, triteia_hip_bmm_2_4 and triteia_hip_sbmm_2_4 called with exactly the reference launchers'
     argument lists (marlin_nm.cu:42-46, triteia_nm_bmm.cu:760-764, triteia_nm_sbmm.cu:809-815), no binding layer."""

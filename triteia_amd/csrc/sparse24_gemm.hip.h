@@ -105,6 +105,11 @@ struct Sparse24Args {
   float* partial;
   long partial_rows;        // rows of one split's block in `partial` (= rows of `out`)
   int ksplit_steps;
+  // A workgroup takes 128 >> sub_shift columns of a column block (0..3): launches of a few dozen workgroups are bound
+  // by what one CU's memory pipeline delivers (about 30 GB/s however many wavefronts and requests it has in flight),
+  // so the same work spread over more CUs is faster.  Each output column is still summed over K by the same wavefronts
+  // in the same order: the bits do not depend on sub_shift.
+  int sub_shift;
 };
 
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
@@ -178,6 +183,10 @@ struct TileCtx {
   int rot;                  // this delta's walk over K starts at step `rot` and wraps around
   int step0;                // first step of this workgroup's share of K (K split across workgroups), else 0
   int cb;                   // column block
+  int ra;                   // the 8-column block (0..15) of the column block whose weights this lane loads: r, or with
+                            // sub_shift > 0 one of the 16 >> sub_shift blocks of this workgroup's share
+  int col0;                 // first column of this workgroup's share inside the column block
+  int nblk_shift;           // log2 of the 8-column blocks in the share (4 - sub_shift)
   int tid, wave, lane, r, q;
   // fused routing (up to kRawParts x 64 tokens, kRawParts per lane): for part j of the batch (tokens
   // 64 j .. 64 j + 63), lane s of raw_list[j] holds the s-th of the group's tokens in that part, and
@@ -254,7 +263,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   // The scales of this thread's 8 output features, for the epilogue: requested here, behind the first
   // weights, so that no wait for them can land ahead of a request (requested before the loop over
   // passes they were waited for at the loop's entry: a full memory round trip before the first weights).
-  const half8_t sv = *reinterpret_cast<const half8_t*>(c.sc + (c.tid & 15) * 8);
+  const half8_t sv = *reinterpret_cast<const half8_t*>(c.sc + c.col0 + (c.tid & ((1 << c.nblk_shift) - 1)) * 8);
 
   // Every lane always loads from a valid address, so that the number of loads per step is
   // fixed and the hardware load counter can be waited on exactly (the output columns of the
@@ -370,7 +379,9 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   for (int nt = 0; nt < NTT; nt++) {
     if (nt * 16 >= cnt) break;
     if (nt > 0) lds_barrier();
-    float* dst = &red[wave][r][32 * q];   // D: lane (n = r, qq = q) owns features 32q + 8j + c
+    // D: lane (n = r, qq = q) owns rows 4q + j of the MFMA, i.e. columns 8 (4q + j) + c of the workgroup's share (rows
+    // past the share, when it is narrower than 128 columns, repeat its blocks and are never read back)
+    float* dst = &red[wave][r][32 * q];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       float4_t lo = {acc[0][nt][j], acc[1][nt][j], acc[2][nt][j], acc[3][nt][j]};
@@ -379,10 +390,10 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
       *reinterpret_cast<float4_t*>(dst + 8 * j + 4) = hi;
     }
     lds_barrier();
-    // 16 tokens x 128 features = 256 chunks of 8 features
-    for (int ch = c.tid; ch < 256; ch += 64 * KW) {
-      const int tok = ch >> 4;
-      const int f0 = (ch & 15) * 8;
+    // 16 tokens x (128 >> sub_shift) features in chunks of 8 features
+    for (int ch = c.tid; ch < (16 << c.nblk_shift); ch += 64 * KW) {
+      const int tok = ch >> c.nblk_shift;
+      const int f0 = (ch & ((1 << c.nblk_shift) - 1)) * 8;
       const int row = s_rows[nt * 16 + tok];
       if (row < 0) continue;
       float v[8];
@@ -397,13 +408,13 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
       }
       if (p.ksplit_steps) {
         // this workgroup's share of K only: the sums go to its block of the partial buffer as they are
-        float* pp = p.partial + ((long)blockIdx.z * p.partial_rows + row) * p.m + c.cb * 128 + f0;
+        float* pp = p.partial + ((long)blockIdx.z * p.partial_rows + row) * p.m + c.cb * 128 + c.col0 + f0;
         *reinterpret_cast<float4_t*>(pp) = float4_t{v[0], v[1], v[2], v[3]};
         *reinterpret_cast<float4_t*>(pp + 4) = float4_t{v[4], v[5], v[6], v[7]};
         continue;
       }
       // (sv: f0 is the same for every chunk of a thread, 64 * KW being a multiple of 16)
-      _Float16* op = p.out + (long)row * p.out_stride + c.cb * 128 + f0;
+      _Float16* op = p.out + (long)row * p.out_stride + c.cb * 128 + c.col0 + f0;
       half8_t old = {0, 0, 0, 0, 0, 0, 0, 0};
       if (p.accumulate) old = *reinterpret_cast<const half8_t*>(op);
       half8_t o;
@@ -429,13 +440,15 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   // Unit = (group, column block).  Workgroups are dealt round-robin to the 8 XCDs (each with
   // its own L2); the column blocks of a group are numbered so that every XCD owns a contiguous
   // run of them: the per-group unit count is padded to a multiple of 8 (padding units exit).
-  const int col_blocks = p.m >> 7;
-  const int cb_pad = (col_blocks + 7) & ~7;
+  // (with sub_shift > 0 the same holds for the shares of column blocks)
+  const int col_units = (p.m >> 7) << p.sub_shift;
+  const int cu_pad = (col_units + 7) & ~7;
   const int unit = blockIdx.x;
-  const int grp = unit / cb_pad;
-  const int i = unit - grp * cb_pad;
-  const int cb = p.xcd_swizzle ? (i & 7) * (cb_pad >> 3) + (i >> 3) : i;
-  if (cb >= col_blocks) return;
+  const int grp = unit / cu_pad;
+  const int i = unit - grp * cu_pad;
+  const int cu = p.xcd_swizzle ? (i & 7) * (cu_pad >> 3) + (i >> 3) : i;
+  if (cu >= col_units) return;
+  const int cb = cu >> p.sub_shift;
 
   TileCtx c;
   c.tid = threadIdx.x;
@@ -444,6 +457,12 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   c.r = c.lane & 15;
   c.q = c.lane >> 4;
   c.cb = cb;
+  c.nblk_shift = 4 - p.sub_shift;
+  {
+    const int sub = cu & ((1 << p.sub_shift) - 1);
+    c.ra = (sub << c.nblk_shift) + (c.r & ((1 << c.nblk_shift) - 1));
+    c.col0 = sub << (7 - p.sub_shift);
+  }
 #pragma unroll
   for (int j = 0; j < kRawParts; j++) c.raw_list[j] = c.raw_before[j] = 0;
   c.raw_before[kRawParts] = 0;
@@ -458,8 +477,8 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   c.mrow = p.m >> 2;
   // everything that depends on the delta: operand pointers and the request for this thread's scales
   auto bind_delta = [&](int delta) {
-    c.qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * c.r;
-    c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.r >> 3)) * 16 + (c.r & 7);
+    c.qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * c.ra;
+    c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.ra >> 3)) * 16 + (c.ra & 7);
     c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;
     // side-by-side deltas start their walks spread around the ring of steps (by the delta's index,
     // so that a result does not depend on where the weights happen to lie in memory)

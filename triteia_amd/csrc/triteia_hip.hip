@@ -60,7 +60,7 @@ struct Knobs {
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
   int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
-  int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1;
+  int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset;
 };
 Knobs g_knobs;
 std::once_flag g_knobs_once;
@@ -76,7 +76,7 @@ void read_knobs() {
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
       {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
       {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
-      {"KSPLIT", &k.ksplit},
+      {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift},
   };
   char name[64];
   for (auto& e : table) {
@@ -146,13 +146,27 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   if (tsplit < 1) tsplit = 1;
   if (tsplit > 65535) tsplit = 65535;
-  const long cb_pad = (a.m / 128 + 7) / 8 * 8;   // column blocks padded to the 8 XCDs
+  // Uniform launches of few workgroups give each workgroup a share of a column block (128 >> sub_shift columns)
+  // instead of a whole one, halving the share while the launch stays within one workgroup per CU: more CUs take part,
+  // and the sums do not change (see Sparse24Args::sub_shift).  The gain is small, because every share still reads all
+  // the activations: 16 tokens on 4096 x 4096 (32 column blocks) 11.4 -> 10.1 us in shares of 16 columns, on 4096 x 11008
+  // (86) 12.4 -> 11.1 us in shares of 64 (in shares of 32, 344 workgroups: 18.2 us); one token on each of 8 matrices of
+  // 4096 x 4096 (256 column blocks already) 13.2 -> 16.5 us in shares of 64, which the rule does not do.
+  const bool uniform = !a.raw_indices && !a.tiles && !a.g_delta;
+  {
+    int s = 0;
+    const long blocks = (long)a.n_groups * (a.m / 128) * tsplit * zsplit;
+    if (uniform && nt == 1 && zsplit == 1)
+      while (s < 3 && (blocks << (s + 1)) <= 256) s++;
+    a.sub_shift = knob_or(knobs().sub_shift, s);
+    if (a.sub_shift < 0 || a.sub_shift > 3) a.sub_shift = 0;
+  }
+  const long cb_pad = (((long)(a.m / 128) << a.sub_shift) + 7) / 8 * 8;   // column shares padded to the 8 XCDs
   // A launch of at most one workgroup per CU runs 8 wavefronts per workgroup with one step in
   // flight each: more waves, not more bytes per wave, is what raises the rate there (measured:
   // cfg1 14.3 -> 13.6 us, 16-token matmul 12.3 -> 11.4 us; 16 wavefronts and two steps per wave are slower).
   // Only for uniform groups (matmul, bmm): the split of K among the wavefronts fixes the order of the
   // fp32 sums, and a routed token must have the same bits whatever the size of its batch.
-  const bool uniform = !a.raw_indices && !a.tiles && !a.g_delta;
   const bool one_per_cu = uniform && zsplit == 1 && (nt == 1 || nt == 2) && (long)a.n_groups * cb_pad * tsplit <= 256;
   const int kw = knob_or(knobs().kw, one_per_cu ? 8 : 4);
   // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight (2 with
