@@ -95,3 +95,41 @@ def test_product_code_never_reaches_for_the_oracle():
             if path.suffix in (".py", ".h", ".hip") and "oracle" in path.read_text(errors="replace"):
                 offenders.append(str(path.relative_to(root)))
     assert not offenders, offenders
+
+
+def test_dispatch_queries_at_the_documented_points():
+    """Which kernel a call would run is a pure host-side function of the shapes and the knobs: the answers at the
+    benchmark's points, as the documentation states them (no GPU involved)."""
+    lib = _ffi.lib()
+    _ffi.reload_env()
+    uniform = lib.triteia_hip_uniform_kernel          # (m, batch, tokens, k, with_scratch)
+    assert uniform(4096, 1, 16, 4096, 1) == 0          # cfg0: K of 4096 is too short for a split across workgroups
+    assert uniform(4096, 8, 1, 4096, 1) == 0           # cfg1: a workgroup per CU already
+    assert uniform(8192, 1, 16, 8192, 1) == 1004       # long K, few workgroups: K split in 4 ...
+    assert uniform(8192, 1, 16, 8192, 0) == 0          # ... only with a scratch buffer
+    assert lib.triteia_hip_bmm_scratch_bytes(8192, 1, 16, 8192) == 4 * 16 * 8192 * 4
+    assert lib.triteia_hip_bmm_scratch_bytes(4096, 1, 16, 4096) == 0
+    assert uniform(4096, 1, 1024, 4096, 1) == 33       # 32-token tiles on eight wavefronts (one workgroup per CU)
+    assert uniform(4096, 1, 1536, 4096, 1) == 65       # 64-token tiles on eight wavefronts
+    assert uniform(4096, 1, 4096, 4096, 1) == 256      # one round of 256-token tiles
+    assert uniform(28672, 1, 4096, 8192, 1) == 64      # several rounds: 64-token tiles, two workgroups per CU
+    assert uniform(4096, 1, 128, 4096, 1) == 0
+    assert uniform(100, 1, 16, 4096, 1) == -1          # not a legal shape
+    routed = lib.triteia_hip_routed_in_kernel          # (tokens, deltas, m, k)
+    assert routed(64, 16, 4096, 4096) == 1             # cfg2: one launch, no plan
+    assert routed(256, 16, 4096, 4096) == 1
+    assert routed(65, 17, 4096, 4096) == 0             # above 64 tokens only up to 16 deltas
+    assert routed(256, 32, 11008, 4096) == 0           # cfg3: planned ...
+    assert lib.triteia_hip_planned_tile_kernel(256, 32, 11008, 4096) == 32   # ... and its 32-token tiles go to the wide kernel
+    assert lib.triteia_hip_planned_tile_kernel(256, 16, 4096, 4096) == 0     # a narrow layer keeps the streaming kernel
+    assert lib.triteia_hip_planned_tile_kernel(1024, 16, 4096, 4096) == 32   # except for a thousand tokens in full tiles
+    assert lib.triteia_hip_plan_tile_tokens(64, 16) == 16
+    assert lib.triteia_hip_plan_tile_tokens(4096, 16) == 64
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode == 2
+    assert "ONE GPU" in res.stderr
