@@ -30,7 +30,7 @@ constexpr int kPlanHeaderInts = 8;
 constexpr int kPlanWideTile = 64;      // tokens per wide tile
 constexpr int kPlanWideMinRest = 33;   // a rest of at least this many tokens still forms a wide tile
 constexpr int kPlanMaxDeltas = 8192;  // per-delta cursors live in LDS
-constexpr int kPlanThreads = 256;
+constexpr int kPlanThreads = 1024;     // 16 wavefronts
 constexpr int kPlanCachedTokens = 8192;  // token indices kept in LDS between the two passes
 constexpr int kPlanMinTile = 16;      // smallest tile size a plan can be built for
 
@@ -72,26 +72,38 @@ __device__ __forceinline__ int wave_excl_scan(int v, int lane, int* total) {
 }
 
 // One workgroup.  indices[t] - index_offset outside [0, n_deltas) means "no delta".
+//
+// The tokens are cut into `shares` of whole 64-token pieces, one per wavefront (as many as the 8192 LDS counters
+// allow: 16 shares up to 512 deltas, one at 8192).  Every token is counted under (share, delta); the scan over the
+// deltas then turns the counts of a delta's shares into the shares' first slots in perm, one behind the other, so
+// that the wavefronts can place their shares side by side and the order inside a delta is still the batch's.
 __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __restrict__ indices, int n_tokens,
                                                                  int n_deltas, int index_offset, int tile, int wide,
                                                                  int* __restrict__ ws) {
-  __shared__ int s_cursor[kPlanMaxDeltas];
+  __shared__ int s_cursor[kPlanMaxDeltas];     // [share][delta]: counts, then cursors into perm
   __shared__ int s_delta[kPlanCachedTokens];   // pass 1 leaves each token's delta here for pass 2
   const PlanLayout L = plan_layout(n_tokens, n_deltas);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
+  const int wave = tid >> 6;
 
-  for (int d = tid; d < n_deltas; d += kPlanThreads) s_cursor[d] = 0;
+  int shares = kPlanThreads / 64;
+  if (n_deltas > 0 && shares > kPlanMaxDeltas / n_deltas) shares = kPlanMaxDeltas / n_deltas;
+  if (shares > (n_tokens + 63) / 64) shares = (n_tokens + 63) / 64;
+  if (shares < 1) shares = 1;
+  const int share_tokens = (((n_tokens + shares - 1) / shares) + 63) & ~63;   // whole 64-token pieces
+
+  for (int i = tid; i < shares * n_deltas; i += kPlanThreads) s_cursor[i] = 0;
   __syncthreads();
   for (int t = tid; t < n_tokens; t += kPlanThreads) {
     int d = indices[t] - index_offset;
     if (d < 0 || d >= n_deltas) d = -1;
     if (t < kPlanCachedTokens) s_delta[t] = d;
-    if (d >= 0) atomicAdd(&s_cursor[d], 1);
+    if (d >= 0) atomicAdd(&s_cursor[(t / share_tokens) * n_deltas + d], 1);
   }
   __syncthreads();
 
-  if (tid < 64) {
+  if (wave == 0) {
     // exclusive scans over the deltas, 64 per iteration: token counts -> first slot in perm,
     // tile counts -> first tile
     int running = 0, tiles = 0, wides = 0, alls = 0, groups = 0;
@@ -100,7 +112,9 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
     int4* all_out = reinterpret_cast<int4*>(ws + L.all);
     for (int base = 0; base < n_deltas; base += 64) {
       const int d = base + lane;
-      const int c = d < n_deltas ? s_cursor[d] : 0;
+      int c = 0;
+      if (d < n_deltas)
+        for (int w = 0; w < shares; w++) c += s_cursor[w * n_deltas + d];
       int chunk_tokens, chunk_tiles, chunk_wides, chunk_alls;
       const int offs = running + wave_excl_scan(c, lane, &chunk_tokens);
       // split this delta's tokens: wide tiles first, the rest in narrow tiles
@@ -131,7 +145,15 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
         }
         alls += chunk_alls;
       }
-      if (d < n_deltas) s_cursor[d] = offs;
+      if (d < n_deltas) {
+        // the shares' pieces of this delta's run of slots, in the order of the shares
+        int before = 0;
+        for (int w = 0; w < shares; w++) {
+          const int mine = s_cursor[w * n_deltas + d];
+          s_cursor[w * n_deltas + d] = offs + before;
+          before += mine;
+        }
+      }
       running += chunk_tokens;
       tiles += chunk_tiles;
       wides += chunk_wides;
@@ -147,11 +169,17 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
       ws[L.header + 6] = 0;
       ws[L.header + 7] = 0;
     }
-    // stable placement: 64 tokens at a time, tokens with equal delta ranked by lane order
-    for (int base = 0; base < n_tokens; base += 64) {
+  }
+  __syncthreads();
+
+  if (wave < shares) {
+    // stable placement of this wavefront's share: 64 tokens at a time, tokens with equal delta ranked by lane order
+    int* cursor = s_cursor + wave * n_deltas;
+    const int end = min(n_tokens, (wave + 1) * share_tokens);
+    for (int base = wave * share_tokens; base < end; base += 64) {
       const int t = base + lane;
       int d = -1;
-      if (t < n_tokens) {
+      if (t < end) {
         if (t < kPlanCachedTokens) {
           d = s_delta[t];
         } else {
@@ -169,11 +197,11 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
       }
       if (d >= 0) {
         const int rank = __popcll(same & ((1ull << lane) - 1ull));
-        const int first = s_cursor[d];
+        const int first = cursor[d];
         ws[L.perm + first + rank] = t;
         // every lane of the group has read the cursor before its first lane moves it
         __builtin_amdgcn_wave_barrier();
-        if (rank == 0) s_cursor[d] = first + __popcll(same);
+        if (rank == 0) cursor[d] = first + __popcll(same);
       }
     }
   }
