@@ -477,6 +477,48 @@ def run_probes(torch, ffi):
                       "gbs": round(nbytes / t_loads / 1e9, 1), "frac_of_8_tbs": round(nbytes / t_loads / 1e9 / HBM_PEAK_GBS, 4)},
            "product_kernel": {"us": round(t_real * 1e6, 2), "gbs": round(nbytes / t_real / 1e9, 1),
                               "frac_of_8_tbs": round(nbytes / t_real / 1e9 / HBM_PEAK_GBS, 4), "frac_of_stream_probe": round(t_loads / t_real, 4)}}
+    # what a launch of the same grid costs when it does nothing, and what a plain read of the same packed weights streams at
+    sink1 = torch.zeros(64, dtype=torch.float32, device="cuda:0")
+    grid = 16 * ((wl.m // 128 + 7) // 8 * 8)
+
+    def floor(_i):
+        prob._chk(lib.triteia_hip_probe_launch(grid, P(sink1), 0, prob.stream()))
+
+    def plain_read(i):
+        q = prob.weights[i % prob.copies][0]
+        prob._chk(lib.triteia_hip_probe_read(P(q), q.numel() * q.element_size(), 2048, P(sink1), 0, prob.stream()))
+
+    def timed_in_a_graph(call, n=40, reps=7):
+        # launches this short are bound by the host when issued one by one: a captured graph of n of them, replayed
+        for i in range(3):
+            call(i)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(n):
+                    call(i)
+        torch.cuda.synchronize()
+        durs = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            e1.synchronize()
+            durs.append(e0.elapsed_time(e1) / n * 1e-3)
+        del graph
+        return float(np.median(durs))
+
+    t_floor, t_read = timed_in_a_graph(floor), timed_in_a_graph(plain_read)
+    q_bytes = prob.weights[0][0].numel() * prob.weights[0][0].element_size()
+    read_gbs = q_bytes / (t_read - t_floor) / 1e9      # the rate of the streaming itself, the launch's own cost taken off
+    out["launch_floor"] = {"kernel": f"launch_floor_kernel, {grid} workgroups of 256 threads", "us": round(t_floor * 1e6, 2)}
+    out["plain_read"] = {"kernel": "stream_read_kernel, 2048 workgroups", "bytes": q_bytes, "us": round(t_read * 1e6, 2),
+                         "gbs_beyond_the_launch": round(read_gbs, 1)}
+    out["product_kernel"]["us_of_a_launch_plus_a_plain_read_of_its_bytes"] = round((t_floor + nbytes / (read_gbs * 1e9)) * 1e6, 2)
     del prob
     torch.cuda.empty_cache()
     src = torch.randn(16384, device="cuda:0").half()

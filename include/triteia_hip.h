@@ -206,6 +206,11 @@ TRITEIA_HIP_API int triteia_hip_routed_in_kernel(int prob_n, int n_deltas, int p
  * triteia_hip_probe_stream: the launch that triteia_hip_sbmm_2_4_routed makes for a batch of at most 64 tokens over
  * at most 16 deltas, with the sparse MFMAs left out: same requests, waits, reduction and stores, meaningless values
  * in C.  What the memory system alone allows for that kernel's access pattern. */
+/* triteia_hip_probe_launch: `workgroups` workgroups of 256 threads that start and end (one thread writes out[0]): the cost
+ * of a launch.  triteia_hip_probe_read: a plain streaming read of `bytes` bytes at `src` (16-byte aligned, a multiple of
+ * 16) by `workgroups` workgroups of 256 threads; `out`: at least 4 bytes of device memory. */
+TRITEIA_HIP_API int triteia_hip_probe_launch(int workgroups, void* out, int dev, void* stream);
+TRITEIA_HIP_API int triteia_hip_probe_read(const void* src, size_t bytes, int workgroups, void* out, int dev, void* stream);
 TRITEIA_HIP_API int triteia_hip_probe_mfma(int variant, int iters, void* out, const void* random_fp16, int dev, void* stream);
 TRITEIA_HIP_API int triteia_hip_probe_stream(const void* A, const void* B, const void* meta, void* C, const void* s, const void* token_indices,
                              int n_deltas, int prob_m, int prob_n, int prob_k, int dev, void* stream);

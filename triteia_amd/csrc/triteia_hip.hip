@@ -677,6 +677,24 @@ int triteia_hip_probe_mfma(int variant, int iters, void* out, const void* random
   return check_launch("mfma_probe_kernel");
 }
 
+int triteia_hip_probe_launch(int workgroups, void* out, int dev, void* stream) {
+  if (workgroups <= 0 || workgroups > (1 << 20) || !out) return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_launch: workgroups=%d or a null buffer", workgroups);
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  hipLaunchKernelGGL(launch_floor_kernel, dim3((unsigned)workgroups), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<float*>(out));
+  return check_launch("launch_floor_kernel");
+}
+
+int triteia_hip_probe_read(const void* src, size_t bytes, int workgroups, void* out, int dev, void* stream) {
+  if (workgroups <= 0 || workgroups > (1 << 20) || !out || !src || bytes % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0)
+    return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_read: needs a 16-byte aligned buffer of a multiple of 16 bytes and 1 .. 2^20 workgroups");
+  DeviceGuard g(dev);
+  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
+  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4_t*>(src), (long)(bytes / 16), static_cast<float*>(out));
+  return check_launch("stream_read_kernel");
+}
+
 int triteia_hip_probe_stream(const void* A, const void* B, const void* meta, void* C, const void* s, const void* token_indices,
                              int n_deltas, int prob_m, int prob_n, int prob_k, int dev, void* stream) {
   if (int e = check_gemm_shape(prob_m, prob_n, prob_k, -1)) return e;

@@ -37,6 +37,8 @@ SIGNATURES = {
     "triteia_hip_sbmm_2_4_planned": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_int, _c_vp]),
     "triteia_hip_sbmm_routed_workspace_bytes": (_c_sz, [_c_int, _c_int]),
     "triteia_hip_plan_tile_tokens": (_c_int, [_c_int, _c_int]),
+    "triteia_hip_probe_launch": (_c_int, [_c_int, _c_vp, _c_int, _c_vp]),
+    "triteia_hip_probe_read": (_c_int, [_c_vp, ctypes.c_size_t, _c_int, _c_vp, _c_int, _c_vp]),
     "triteia_hip_probe_mfma": (_c_int, [_c_int, _c_int, _c_vp, _c_vp, _c_int, _c_vp]),
     "triteia_hip_probe_stream": (_c_int, [_c_vp] * 6 + [_c_int] * 4 + [_c_int, _c_vp]),
     "triteia_hip_routed_in_kernel": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
