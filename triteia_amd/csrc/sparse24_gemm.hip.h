@@ -498,29 +498,35 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
     // instead of a separate routing launch and a dependent descriptor read.
     int d[kRawParts];     // this lane's tokens: lane, 64 + lane, ...
 #pragma unroll
-    for (int j = 0; j < kRawParts; j++) d[j] = (64 * j + c.lane < p.raw_count) ? p.raw_indices[64 * j + c.lane] : -1;
+    // (every lane loads from a valid address, the last index standing in for those past the end: loads under a branch
+    // make the compiler wait for everything in flight -- the weights requested below included -- before the first use
+    // of an index, instead of for the indices alone)
+    for (int j = 0; j < kRawParts; j++) d[j] = p.raw_indices[min(64 * j + c.lane, p.raw_count - 1)];
     if (EAGER) {
       // group g is delta g: its first weights are requested right behind the indices
       if (grp >= p.n_deltas) return;
       delta = grp;
       bind_delta(delta);
-      // (only the workgroup that takes a group's first tokens: the others of a launch that splits a group's tokens over
-      // blockIdx.y mostly find nothing to do, and a prefetched step each would be traffic for nothing)
-      if (blockIdx.y == 0) {
+      // Only the workgroup that takes a group's first tokens needs them: the others of a launch that splits a group's
+      // tokens over blockIdx.y mostly find nothing to do, and a step each would be traffic for nothing.  They issue the
+      // same loads on packed row 0 instead (one hot piece per column block), because requests under a branch would make
+      // the compiler wait for everything in flight before the first use of an index: where two paths meet it assumes
+      // the shorter queue, and "all but the newest 0" then includes these weights, a cold round trip to HBM, ahead of
+      // the routing.
+      const bool lead = blockIdx.y == 0;
 #pragma unroll
-        for (int j = 0; j < NPRE; j++) {
-          const int st = c.wave + j * KW;              // this wave's j-th step (beyond the end of K: loads go unused)
-          int ps = st + c.rot;
-          if (ps >= c.n_steps) ps -= c.n_steps;
-          if (st >= c.n_steps) ps = 0;
-          const int tr = min((ps << 2) + c.q, c.k_rows - 1);
-          const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
-          const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
+      for (int j = 0; j < NPRE; j++) {
+        const int st = c.wave + j * KW;              // this wave's j-th step (beyond the end of K: loads go unused)
+        int ps = st + c.rot;
+        if (ps >= c.n_steps) ps -= c.n_steps;
+        if (st >= c.n_steps) ps = 0;
+        const int tr = lead ? min((ps << 2) + c.q, c.k_rows - 1) : 0;
+        const uint4_t* wp = c.qw_lane + (long)tr * c.qrow;
+        const uint4_t* mp = c.mt_lane + (long)tr * c.mrow;
 #pragma unroll
-          for (int a = 0; a < 4; a++) pre[j].wq[a] = wp[a];
-          pre[j].mt[0] = mp[0];
-          pre[j].mt[1] = mp[8];
-        }
+        for (int a = 0; a < 4; a++) pre[j].wq[a] = wp[a];
+        pre[j].mt[0] = mp[0];
+        pre[j].mt[1] = mp[8];
       }
       // nothing that needs the indices may be scheduled (with its wait) ahead of these requests
       __builtin_amdgcn_sched_barrier(0);
