@@ -601,25 +601,32 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   }
 
   // blockIdx.y splits a group's tokens between workgroups (each re-streams the weights)
-  bool first_pass = true;
-  for (int t0 = blockIdx.y * 16 * NT; t0 < count; t0 += gridDim.y * 16 * NT) {
+  int t0 = blockIdx.y * 16 * NT;
+  if (EAGER && blockIdx.y == 0 && t0 < count) {
+    // The pass that uses the weights requested ahead of the routing stands on its own, ahead of the loop over the
+    // other passes: inside that loop the compiler has to keep `pre` alive for every iteration, cannot let the K loop's
+    // ring take over its registers, and copies it into the ring instead -- with a wait for those weights, a cold round
+    // trip to HBM, ahead of the first activation request (measured: 1.8 us between the routing and that request).
     const int cnt = min(count - t0, 16 * NT);
-    if (EAGER && first_pass && blockIdx.y == 0) {
-      if (NT == 1 || cnt <= 16) {
-        tile_pass<1, KW, (NT == 1 ? DEPTH : 2), NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
-      } else if (NT == 2 || cnt <= 32) {
-        tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
-      } else {
-        tile_pass<NT, KW, DEPTH, NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
-      }
-    } else if (NT == 1 || cnt <= 16) {
+    if (NT == 1 || cnt <= 16) {
+      tile_pass<1, KW, (NT == 1 ? DEPTH : 2), NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
+    } else if (NT == 2 || cnt <= 32) {
+      tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
+    } else {
+      tile_pass<NT, KW, DEPTH, NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
+    }
+    t0 += gridDim.y * 16 * NT;
+    if (t0 < count) lds_barrier();    // the next pass over this group's tokens reuses s_rows / red
+  }
+  for (; t0 < count; t0 += gridDim.y * 16 * NT) {
+    const int cnt = min(count - t0, 16 * NT);
+    if (NT == 1 || cnt <= 16) {
       tile_pass<1, KW, (NT == 1 ? DEPTH : 2), 0, PROBE>(p, c, start + t0, cnt, red, s_rows);
     } else if (NT == 2 || cnt <= 32) {
       tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), 0, PROBE>(p, c, start + t0, cnt, red, s_rows);
     } else {
       tile_pass<NT, KW, DEPTH, 0, PROBE>(p, c, start + t0, cnt, red, s_rows);
     }
-    first_pass = false;
     // the next pass over this group's tokens reuses s_rows / red
     if (t0 + gridDim.y * 16 * NT < count) lds_barrier();
   }
