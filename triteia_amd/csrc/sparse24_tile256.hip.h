@@ -344,13 +344,19 @@ __global__ __launch_bounds__(512, 1) void sparse24_tile256_kernel(const Sparse24
     const int slot = tq * 64 + nt * 16 + r;
     if (slot >= cnt) continue;
     _Float16* op = p.out + (long)s_rows[slot] * p.out_stride + cb * 128 + 32 * q;
+    // (when the sums are added to what is there: a token's four pieces are requested together, ahead of the arithmetic)
+    half8_t olds[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) olds[j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (p.accumulate) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) olds[j] = *reinterpret_cast<const half8_t*>(op + 8 * j);
+    }
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      half8_t old = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (p.accumulate) old = *reinterpret_cast<const half8_t*>(op + 8 * j);
       half8_t o;
 #pragma unroll
-      for (int c = 0; c < 8; c++) o[c] = scaled_sum_f16(old[c], acc[c][nt][j], sv[j][c]);
+      for (int c = 0; c < 8; c++) o[c] = scaled_sum_f16(olds[j][c], acc[c][nt][j], sv[j][c]);
       *reinterpret_cast<half8_t*>(op + 8 * j) = o;
     }
   }

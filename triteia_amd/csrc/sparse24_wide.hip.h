@@ -276,6 +276,22 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   half8_t sv[4];
 #pragma unroll
   for (int j = 0; j < 4; j++) sv[j] = *reinterpret_cast<const half8_t*>(sc + 8 * j);
+  // (when the sums are added to what is there: all of it is requested at once, ahead of the arithmetic -- one round
+  // trip for the tile instead of one per 8 columns; slots past the end of the tile repeat its last row, a valid address)
+  half8_t olds[NT][4];
+  if (p.accumulate) {
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const _Float16* op = p.out + (long)s_rows[nt * 16 + r] * p.out_stride + cb * 128 + 32 * q;
+#pragma unroll
+      for (int j = 0; j < 4; j++) olds[nt][j] = *reinterpret_cast<const half8_t*>(op + 8 * j);
+    }
+  } else {
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) olds[nt][j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  }
 #pragma unroll
   for (int nt = 0; nt < NT; nt++) {
     const int slot = nt * 16 + r;
@@ -283,11 +299,9 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
     _Float16* op = p.out + (long)s_rows[slot] * p.out_stride + cb * 128 + 32 * q;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      half8_t old = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (p.accumulate) old = *reinterpret_cast<const half8_t*>(op + 8 * j);
       half8_t o;
 #pragma unroll
-      for (int cc = 0; cc < 8; cc++) o[cc] = scaled_sum_f16(old[cc], acc[cc][nt][j], sv[j][cc]);
+      for (int cc = 0; cc < 8; cc++) o[cc] = scaled_sum_f16(olds[nt][j][cc], acc[cc][nt][j], sv[j][cc]);
       *reinterpret_cast<half8_t*>(op + 8 * j) = o;
     }
   }
