@@ -622,7 +622,11 @@ def test_route_plan_is_a_stable_grouping():
     from triteia_amd.python.capi import _ffi, route_plan
     say("route plan")
     rng = np.random.default_rng(51)
-    for T, N, off in [(1, 1, 0), (64, 16, 0), (200, 7, 0), (1000, 300, 0), (130, 5, 3), (70, 100, 0), (700, 3, 0), (520, 40, 0)]:
+    # (the later cases walk through the numbers of token shares the plan kernel places side by side: 16 up to 512
+    # deltas, fewer above, one at 8192; shares of ragged size; more tokens than it keeps in LDS between its passes)
+    for T, N, off in [(1, 1, 0), (64, 16, 0), (200, 7, 0), (1000, 300, 0), (130, 5, 3), (70, 100, 0), (700, 3, 0), (520, 40, 0),
+                      (4096, 16, 0), (65, 2, 0), (129, 513, 0), (5000, 600, 0), (3000, 1024, 2), (2500, 3000, 0), (1500, 8192, 0),
+                      (9000, 4, 0), (8193, 33, 1)]:
         idx = rng.integers(-1, N + off, size=T).astype(np.int32)
         plan = route_plan(torch.from_numpy(idx).to(DEV), N, index_offset=off).cpu().numpy()
         d = idx - off
