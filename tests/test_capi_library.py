@@ -119,6 +119,10 @@ def test_dispatch_queries_at_the_documented_points():
     assert routed(64, 16, 4096, 4096) == 1             # cfg2: one launch, no plan
     assert routed(256, 16, 4096, 4096) == 1
     assert routed(65, 17, 4096, 4096) == 0             # above 64 tokens only up to 16 deltas
+    assert routed(64, 32, 4096, 4096) == 1             # a small layer: the plan's launch would not pay
+    assert routed(64, 32, 11008, 4096) == 0            # 33 .. 64 tokens over many deltas of a large layer: planned ...
+    assert lib.triteia_hip_plan_tile_tokens(64, 32) == 32   # ... in 32-token tiles (a skewed batch's hot delta in one tile)
+    assert routed(32, 32, 11008, 4096) == 1
     assert routed(256, 32, 11008, 4096) == 0           # cfg3: planned ...
     assert lib.triteia_hip_planned_tile_kernel(256, 32, 11008, 4096) == 32   # ... and its 32-token tiles go to the wide kernel
     assert lib.triteia_hip_planned_tile_kernel(256, 16, 4096, 4096) == 0     # a narrow layer keeps the streaming kernel

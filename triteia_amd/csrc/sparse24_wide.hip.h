@@ -276,32 +276,28 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   half8_t sv[4];
 #pragma unroll
   for (int j = 0; j < 4; j++) sv[j] = *reinterpret_cast<const half8_t*>(sc + 8 * j);
-  // (when the sums are added to what is there: all of it is requested at once, ahead of the arithmetic -- one round
-  // trip for the tile instead of one per 8 columns; slots past the end of the tile repeat its last row, a valid address)
-  half8_t olds[NT][4];
-  if (p.accumulate) {
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      const _Float16* op = p.out + (long)s_rows[nt * 16 + r] * p.out_stride + cb * 128 + 32 * q;
-#pragma unroll
-      for (int j = 0; j < 4; j++) olds[nt][j] = *reinterpret_cast<const half8_t*>(op + 8 * j);
-    }
-  } else {
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) olds[nt][j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-  }
 #pragma unroll
   for (int nt = 0; nt < NT; nt++) {
     const int slot = nt * 16 + r;
     if (slot >= cnt) continue;
     _Float16* op = p.out + (long)s_rows[slot] * p.out_stride + cb * 128 + 32 * q;
+    // (when the sums are added to what is there: a token's four pieces are requested together, ahead of the arithmetic
+    // -- one round trip per 16-token tile instead of one per 8 columns.  All tiles at once would be one round trip in
+    // all, but holds 16 registers per tile, which the 64-token builds do not have.)
+    constexpr bool TOGETHER = !(TOK == 64 && KS == 2);   // (that build is out of registers as it is)
+    half8_t olds[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) olds[j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (TOGETHER && p.accumulate) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) olds[j] = *reinterpret_cast<const half8_t*>(op + 8 * j);
+    }
 #pragma unroll
     for (int j = 0; j < 4; j++) {
+      if (!TOGETHER && p.accumulate) olds[j] = *reinterpret_cast<const half8_t*>(op + 8 * j);
       half8_t o;
 #pragma unroll
-      for (int cc = 0; cc < 8; cc++) o[cc] = scaled_sum_f16(olds[nt][j][cc], acc[cc][nt][j], sv[j][cc]);
+      for (int cc = 0; cc < 8; cc++) o[cc] = scaled_sum_f16(olds[j][cc], acc[cc][nt][j], sv[j][cc]);
       *reinterpret_cast<half8_t*>(op + 8 * j) = o;
     }
   }

@@ -597,7 +597,13 @@ size_t triteia_hip_sbmm_routed_workspace_bytes(int prob_n, int n_deltas) {
 }
 
 int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas) {
-  return 16 * pick_nt(prob_n, prob_n < n_deltas ? prob_n : n_deltas);
+  const int groups = prob_n < n_deltas ? prob_n : n_deltas;
+  int nt = pick_nt(prob_n, groups);
+  // A plan for 33 .. 64 tokens over more than 16 deltas: under a skewed routing the hot delta has more than 16 tokens,
+  // and a second 16-token tile streams its weights again (64 tokens, Zipf(1.2) over 32 deltas: 11008 x 4096 70.5 us in
+  // 16-token tiles, 65.6 in 32-token tiles, 64.0 in 64-token tiles; 4096 x 11008 59.5 / 58.9 / 70.8 us).
+  if (nt == 1 && prob_n > 32 && groups > 16 && knobs().nt == 0) nt = 2;
+  return 16 * nt;
 }
 
 // A plan carries wide (64-token) tiles, next to a narrow-only cut of the same tokens, for batches
@@ -648,6 +654,15 @@ static bool routed_eager_ok(int prob_n, int n_deltas) {
   return n_deltas <= 16 && prob_n >= (prob_n > 64 ? 4 : 2) * n_deltas && knobs().eager;
 }
 static bool routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
+  // (more than 32 tokens over more than 16 deltas of a large layer: a skewed batch then has a delta with several
+  // 16-token passes, which a plan spreads over workgroups while the in-kernel form runs them one after the other, and
+  // the plan's launch is small against the kernel.  64 tokens, Zipf(1.2): 32 deltas of 4096 x 11008 63 -> 58 us,
+  // of 11008 x 4096 69 -> 64 us, 64 deltas of 8192 x 28672 375 -> 352 us; on 4096 x 4096 the in-kernel form stays ahead,
+  // 30.6 against 32-33 us)
+  // (knob fused_route = 2: in the kernel wherever the kernel can -- at most 64 tokens over at most 64 deltas, at most
+  // 256 over at most 32 -- whatever the rules below say; for measurements)
+  if (knobs().fused_route == 2) return prob_n <= kFusedMaxTokens && n_deltas <= (prob_n > 64 ? 32 : 64);
+  if (prob_n > 32 && !routed_eager_ok(prob_n, n_deltas) && (long)prob_k * prob_m >= (1L << 25)) return false;
   return prob_n <= knob_or(knobs().fused_max_tokens, kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
          n_deltas <= (prob_n > 64 ? 16 : 64) && knobs().fused_route &&
          !(prob_n >= 128 && ((!routed_eager_ok(prob_n, n_deltas) && mid_tiles(prob_n, n_deltas, prob_m, prob_k)) ||
