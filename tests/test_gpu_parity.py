@@ -527,6 +527,7 @@ def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, 
     (600, 40, 256, 512, 105, "100000"),    # whatever the bar for the wide tiles says
     (600, 6, 256, 640, 106, "1"),          # a plan of 64-token tiles: the 64-token build takes its narrow-only list
     (200, 3, 128, 256, 107, "200"),        # the same without wide tiles in the plan
+    (150, 5, 640, 384, 108, "200"),        # five K steps: the ring of four stages does not end on a whole turn
 ])
 def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, seed, wide_bar):
     """A plan's 32-token tiles on a wide layer run on the 32-token build of the wide kernel (forced here

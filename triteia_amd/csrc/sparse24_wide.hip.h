@@ -18,6 +18,8 @@
 // distinct banks while every direct-to-LDS load still writes 1 KB of consecutive LDS.
 // Needs k % 128 == 0 (a direct load cannot zero-fill a partial K step).
 #pragma once
+#include <type_traits>
+
 #include "sparse24_gemm.hip.h"
 
 namespace triteia_hip {
@@ -127,11 +129,13 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   // weights requested a moment ago included) once per K step.  The LDS address of a request is
   // M0 + 16 * lane; M0 is an input operand of the statement, so the compiler writes it and knows it is live.
   const uint32_t lds_x_wave = (uint32_t)(uintptr_t)&xs[kh][0][4 * wave][0];
-  auto issue_x = [&](int st) {
+  // (`nta`: the 16-token tiles that hold tokens; the others are neither fetched nor multiplied)
+  auto issue_x = [&](int st, int nta) {   // (nta: a constant where this is called)
     const int stc = min(step0 + min(st, n_steps - 1), all_steps - 1);   // past the end: refetch a valid tile (never read)
     const int stage = st & (kWideStages - 1);
 #pragma unroll
     for (int ii = 0; ii < NT; ii++) {
+      if (ii >= nta) break;
       const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_x_wave + (stage * TOK + 16 * ii) * 256);
       const _Float16* base = p.x + stc * 128;
       asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(xoff[ii]), "s"(base), "{m0}"(dst) : "memory");
@@ -172,7 +176,8 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
     const uint8_t_v bb = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     return __builtin_bit_cast(half16_t, bb);
   };
-  auto compute_step = [&](const WFrag& f, int stage) {
+  auto compute_step = [&](const WFrag& f, int stage, auto nta) {
+    constexpr int NTA = decltype(nta)::value;
     // Per k-half u and per half of the 8 columns: dequantise 4 weight fragments, then run them
     // against the four 16-token B fragments.  B fragments are read one ahead of the MFMAs that
     // use them, so that the LDS latency hides behind 4 MFMAs instead of stalling in front of them.
@@ -196,11 +201,11 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
           A[w] = __builtin_bit_cast(half8_t, av);
         }
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
+        for (int nt = 0; nt < NTA; nt++) {
           half16_t b;
           if (DEPTH < 2) {
             b = b_nxt;
-            if (nt + 1 < NT) b_nxt = read_b(stage, nt + 1, u);
+            if (nt + 1 < NTA) b_nxt = read_b(stage, nt + 1, u);
             else if (b2 == 0) b_nxt = read_b(stage, 0, u);
             else if (u == 0) b_nxt = read_b(stage, 0, 1);
           } else {
@@ -229,24 +234,73 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   // requests each) and DEPTH sets of weights (6 each); the barrier then makes all four waves' parts visible and
   // also says that tile st-1 has been read by everyone, so its stage can be refilled.
   WFrag ring[DEPTH];
-  issue_x(0);
-  issue_x(1);
-  issue_x(2);
+  auto k_loop = [&](auto nta) {
+    constexpr int NTA = decltype(nta)::value;
+    issue_x(0, NTA);
+    issue_x(1, NTA);
+    issue_x(2, NTA);
 #pragma unroll
-  for (int j = 0; j < DEPTH; j++) load_w(ring[j], j);
-  constexpr int TURN = DEPTH > 4 ? DEPTH : 4;   // whole ring turns of both rings (DEPTH divides 4)
-  for (int s0 = 0; s0 < loop_steps; s0 += TURN) {
+    for (int j = 0; j < DEPTH; j++) load_w(ring[j], j);
+    constexpr int TURN = DEPTH > 4 ? DEPTH : 4;   // whole ring turns of both rings (DEPTH divides 4)
+    // Whole turns run without a condition around the arithmetic (a wavefront past the last column block works on
+    // the block before it and stores nothing): behind a skipped step the compiler has to assume that step's weights
+    // still in flight and waits for everything before it requests the next ones.
+    const int whole = n_steps / TURN * TURN;
+    for (int s0 = 0; s0 < whole; s0 += TURN) {
 #pragma unroll
-    for (int j = 0; j < TURN; j++) {
-      const int st = s0 + j;
-      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NT + 6 * DEPTH) : "memory");
-      lds_barrier();
-      if (st < n_steps && active) compute_step(ring[j % DEPTH], j & (kWideStages - 1));
-      issue_x(st + 3);
-      load_w(ring[j % DEPTH], st + DEPTH);
+      for (int j = 0; j < TURN; j++) {
+        const int st = s0 + j;
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NTA + 6 * DEPTH) : "memory");
+        lds_barrier();
+        compute_step(ring[j % DEPTH], j & (kWideStages - 1), nta);
+        __builtin_amdgcn_sched_barrier(0);   // (requests stay behind the step's arithmetic, where its registers are free)
+        issue_x(st + 3, NTA);
+        load_w(ring[j % DEPTH], st + DEPTH);
+      }
     }
+    if (whole < n_steps) {
+#pragma unroll
+      for (int j = 0; j < TURN; j++) {
+        const int st = whole + j;
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NTA + 6 * DEPTH) : "memory");
+        lds_barrier();
+        if (st < n_steps) compute_step(ring[j % DEPTH], j & (kWideStages - 1), nta);
+        issue_x(st + 3, NTA);
+        load_w(ring[j % DEPTH], st + DEPTH);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive the block's LDS
+  };
+  // A plan's tiles are often far from full (a delta with a handful of tokens): a tile whose tokens fit the first half of
+  // its 16-token tiles walks K in a copy of the loop that leaves the other half out (the matrix cores, not the weight
+  // stream, bound a CU that holds three such workgroups).  The count is the same for the whole workgroup.
+  if constexpr (PLAN_ALL) {
+    static_assert(!PLAN_ALL || KS == 1, "the loop below walks all of K");
+    if (cnt <= TOK / 2)
+      k_loop(std::integral_constant<int, NT / 2>{});
+    else
+      k_loop(std::integral_constant<int, NT>{});
+  } else {
+    constexpr std::integral_constant<int, NT> all{};
+    issue_x(0, NT);
+    issue_x(1, NT);
+    issue_x(2, NT);
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) load_w(ring[j], j);
+    constexpr int TURN = DEPTH > 4 ? DEPTH : 4;
+    for (int s0 = 0; s0 < loop_steps; s0 += TURN) {
+#pragma unroll
+      for (int j = 0; j < TURN; j++) {
+        const int st = s0 + j;
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NT + 6 * DEPTH) : "memory");
+        lds_barrier();
+        if (st < n_steps && active) compute_step(ring[j % DEPTH], j & (kWideStages - 1), all);
+        issue_x(st + 3, NT);
+        load_w(ring[j % DEPTH], st + DEPTH);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no direct load may outlive the block's LDS
 
   if (KS == 2) {
     // the second half's sums go to the first half through the memory of the activation rings (same size:
