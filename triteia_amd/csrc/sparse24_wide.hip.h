@@ -230,8 +230,8 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   // step issues its activation tile first and its weights last, so the compiler's wait for the weights of
   // step st ("all but the newest 6 (DEPTH - 1) requests") is exact for DEPTH = 2: the weights of step
   // st + 1 stay in flight across the step.  The hand-written wait at the top of a step says that this
-  // wave's part of tile st has landed: behind it in the queue are at most the tiles st+1, st+2 (NT
-  // requests each) and DEPTH sets of weights (6 each); the barrier then makes all four waves' parts visible and
+  // wave's part of tile st has landed: behind it in the queue are at most the tiles st+1, st+2 (one
+  // request per occupied 16-token tile each) and DEPTH sets of weights (6 each); the barrier then makes all four waves' parts visible and
   // also says that tile st-1 has been read by everyone, so its stage can be refilled.
   WFrag ring[DEPTH];
   auto k_loop = [&](auto nta) {
@@ -245,7 +245,9 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
     // Whole turns run without a condition around the arithmetic (a wavefront past the last column block works on
     // the block before it and stores nothing): behind a skipped step the compiler has to assume that step's weights
     // still in flight and waits for everything before it requests the next ones.
-    const int whole = n_steps / TURN * TURN;
+    // (with K halved inside the workgroup the second half can be a step shorter: both halves run the same
+    // number of barriers, so the unconditional part covers the steps that both have)
+    const int whole = (KS == 1 ? all_steps : all_steps - loop_steps) / TURN * TURN;
     for (int s0 = 0; s0 < whole; s0 += TURN) {
 #pragma unroll
       for (int j = 0; j < TURN; j++) {
@@ -258,10 +260,10 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
         load_w(ring[j % DEPTH], st + DEPTH);
       }
     }
-    if (whole < n_steps) {
+    for (int s0 = whole; s0 < loop_steps; s0 += TURN) {
 #pragma unroll
       for (int j = 0; j < TURN; j++) {
-        const int st = whole + j;
+        const int st = s0 + j;
         asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NTA + 6 * DEPTH) : "memory");
         lds_barrier();
         if (st < n_steps) compute_step(ring[j % DEPTH], j & (kWideStages - 1), nta);
@@ -274,33 +276,10 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   // A plan's tiles are often far from full (a delta with a handful of tokens): a tile whose tokens fit the first half of
   // its 16-token tiles walks K in a copy of the loop that leaves the other half out (the matrix cores, not the weight
   // stream, bound a CU that holds three such workgroups).  The count is the same for the whole workgroup.
-  if constexpr (PLAN_ALL) {
-    static_assert(!PLAN_ALL || KS == 1, "the loop below walks all of K");
-    if (cnt <= TOK / 2)
-      k_loop(std::integral_constant<int, NT / 2>{});
-    else
-      k_loop(std::integral_constant<int, NT>{});
-  } else {
-    constexpr std::integral_constant<int, NT> all{};
-    issue_x(0, NT);
-    issue_x(1, NT);
-    issue_x(2, NT);
-#pragma unroll
-    for (int j = 0; j < DEPTH; j++) load_w(ring[j], j);
-    constexpr int TURN = DEPTH > 4 ? DEPTH : 4;
-    for (int s0 = 0; s0 < loop_steps; s0 += TURN) {
-#pragma unroll
-      for (int j = 0; j < TURN; j++) {
-        const int st = s0 + j;
-        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NT + 6 * DEPTH) : "memory");
-        lds_barrier();
-        if (st < n_steps && active) compute_step(ring[j % DEPTH], j & (kWideStages - 1), all);
-        issue_x(st + 3, NT);
-        load_w(ring[j % DEPTH], st + DEPTH);
-      }
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  }
+  if (PLAN_ALL && cnt <= TOK / 2)
+    k_loop(std::integral_constant<int, NT / 2>{});
+  else
+    k_loop(std::integral_constant<int, NT>{});
 
   if (KS == 2) {
     // the second half's sums go to the first half through the memory of the activation rings (same size:
