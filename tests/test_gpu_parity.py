@@ -528,6 +528,7 @@ def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, 
     (600, 6, 256, 640, 106, "1"),          # a plan of 64-token tiles: the 64-token build takes its narrow-only list
     (200, 3, 128, 256, 107, "200"),        # the same without wide tiles in the plan
     (150, 5, 640, 384, 108, "200"),        # five K steps: the ring of four stages does not end on a whole turn
+    (2600, 10, 640, 384, 109, "200"),     # a plan of 64-token tiles, full and ragged (halves with 32, a few and no tokens)
 ])
 def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, seed, wide_bar):
     """A plan's 32-token tiles on a wide layer run on the 32-token build of the wide kernel (forced here
@@ -559,8 +560,16 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     check_close(got, ref, what="32-token wide kernel")
     assert not torch.equal(outs["1"], outs["0"]) or k <= 128, "the knob did not change the kernel"
     assert float((outs["1"].float() - outs["0"].float()).norm()) <= 1e-3 * float(outs["0"].float().norm())
-    # accumulate in place on top of a base
+    # two steps of weights in flight (64-token tiles taken as two halves by the 32-token build): every token's sum
+    # over K is formed in the same order
     setknob(monkeypatch, "TRITEIA_HIP_MID", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_MID_DEPTH", "2")
+    out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
+    sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
+    torch.cuda.synchronize()
+    assert torch.equal(out, outs["1"]), "the two-deep build changed bits"
+    setknob(monkeypatch, "TRITEIA_HIP_MID_DEPTH", "1")
+    # accumulate in place on top of a base
     base = torch.from_numpy(activations(T, m, seed + 3)).to(DEV)
     acc = base.clone()
     sbmm_2_4_routed(gx, gq, gm, acc, gs, gi, accumulate=True)

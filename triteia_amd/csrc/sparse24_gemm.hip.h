@@ -110,6 +110,9 @@ struct Sparse24Args {
   // so the same work spread over more CUs is faster.  Each output column is still summed over K by the same wavefronts
   // in the same order: the bits do not depend on sub_shift.
   int sub_shift;
+  // 1: the plan's tiles hold up to 64 tokens and the 32-token build of the wide kernel takes each as two halves
+  // (workgroups 2g and 2g + 1 of a column group; a half without tokens returns at once)
+  int tile_halves;
 };
 
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }

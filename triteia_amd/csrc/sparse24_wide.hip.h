@@ -53,8 +53,13 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   const int cgs = (col_blocks + 3) >> 2;
   const int cg_pad = (cgs + 7) & ~7;
   const int unit = blockIdx.x;
-  const int grp = unit / cg_pad;
+  int grp = unit / cg_pad;
   const int i = unit - grp * cg_pad;
+  int half = 0;
+  if (PLAN_ALL && TOK == 32 && p.tile_halves) {
+    half = grp & 1;
+    grp >>= 1;
+  }
   const int cg = p.xcd_swizzle ? (i & 7) * (cg_pad >> 3) + (i >> 3) : i;
   if (cg >= cgs) return;
   int delta, start, count;
@@ -71,8 +76,8 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
       }
     }
     delta = d.x;
-    start = d.y;
-    count = d.z;
+    start = d.y + 32 * half;
+    count = d.z - 32 * half;
   } else {
     const int chunks = (p.uniform_count + TOK - 1) / TOK;
     const int gi = grp / chunks, tc = grp - gi * chunks;

@@ -58,7 +58,7 @@ struct Knobs {
   int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
-  int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1;
+  int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
   int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset;
 };
@@ -74,7 +74,7 @@ void read_knobs() {
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
       {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
-      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
+      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
       {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
       {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift},
   };
@@ -623,6 +623,29 @@ constexpr int kPlanWideMinUnits = 150;
 // 24.9 -> 42.4 us).  The host only has the upper bound on the tiles; 600 on that bound separates the measured cases.
 constexpr int kMidMinUnits = 480;
 constexpr int kMidNarrowMinUnits = 280, kMidNarrowMinUnits64 = 150, kMidNarrowMinTokens = 768, kMidNarrowMaxTokens = 2048;
+// A plan launch of at most two workgroups per CU (in 32-token tiles x 512-column groups, on the plan's upper bound of
+// tiles) runs on the 32-token build with two steps of weights in flight per wavefront, a 64-token plan tile as two
+// halves: with so few wavefronts per SIMD one step in flight leaves the memory latency of every step in the open.
+// Measured with evenly routed batches of 256 .. 2048 tokens over 4 .. 32 deltas (against one step in flight / against
+// what the rules chose before): 16 deltas of 4096 x 4096 with 768 / 1024 / 1536 tokens 43.5 / 43.9 -> 39.3, 47.5 / 47.8 ->
+// 42.3, 57.3 / 59.4 -> 55.0 us; 8 of 8192 x 8192 with 512 tokens 83.2 / 93.5 -> 74.6; 4 of 4096 x 11008 with 512 tokens
+// 52.8 / 60.7 -> 50.2; 32 of 11008 x 4096 with 1024 tokens 126.8 / 130.0 -> 117.1 us; with randomly routed batches the
+// gain is 4-10 % (16 deltas of 4096 x 4096 with 768 / 1024 tokens 49.6 -> 45.0, 57.0 -> 54.7 us).  Past two workgroups
+// per CU the third workgroup of the one-deep build is worth more (16 deltas of 4096 x 4096 with 2048 randomly routed
+// tokens, 640 units on the bound: 76.2 -> 84.8 us; 4 / 8 of 4096 x 11008 with 768 tokens 66.5 -> 77.4, 73.6 -> 83.6 us), so
+// the bound itself must fit; below 288 units the K-split narrow kernel is faster (16 deltas of 4096 x 4096 with 512
+// tokens 33.3 against 40.5 us), and so it is with few tokens per tile (256 tokens, Zipf(1.2) over 32 deltas of
+// 11008 x 4096, 6.4 per tile on the bound: 89.6 against 102.6 us).
+constexpr long kMidDeepMinUnits = 288, kMidDeepMaxUnits = 512, kMidDeepMinTokensPerTile = 12;
+static long mid_units32(int prob_n, int n_deltas, int prob_m, int tile) {
+  const long cgs = (prob_m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
+  return (long)plan_max_tiles(prob_n, n_deltas, tile) * (tile == 64 ? 2 : 1) * cg_pad;
+}
+static bool mid_deep(int prob_n, int n_deltas, int prob_m, int tile) {
+  const int forced = knobs().mid_depth;
+  if (forced == 1 || forced == 2) return forced == 2;
+  return mid_units32(prob_n, n_deltas, prob_m, tile) <= kMidDeepMaxUnits;
+}
 static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   const int tile = triteia_hip_plan_tile_tokens(prob_n, n_deltas);
   // (64-token plans as well, on the 64-token build, where K is short: cfg3 at 1024 / 2048 tokens 196 -> 170 /
@@ -636,6 +659,11 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   // tile on the bound, 128 tokens over 32 deltas of 4096 x 11008, it depends on the routing: 82 -> 92 us under Zipf(1.0),
   // 76 -> 66 us under Zipf(1.2))
   if (2 * (long)prob_n < (long)knobs().mid_min_half_tokens * tiles) return false;
+  if (tile == 32 || tile == 64) {
+    const long u32 = mid_units32(prob_n, n_deltas, prob_m, tile);
+    if (knobs().mid_depth != 1 && u32 >= kMidDeepMinUnits && u32 <= kMidDeepMaxUnits && prob_n >= kMidDeepMinTokensPerTile * tiles)
+      return true;
+  }
   const long cgs = (prob_m / 128 + 3) / 4;
   if (cgs < knobs().mid_min_column_groups) {
     // A layer of fewer than 16 column groups (m = 4096): with few tokens per tile it is even at best (64 deltas with 8
@@ -811,7 +839,13 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
   if (mid) {
     const long cgs = (a.m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
     if ((long)a.n_groups * cg_pad > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units");
-    if (tile == 32)
+    const long units32 = (long)a.n_groups * (tile == 64 ? 2 : 1) * cg_pad;   // in 32-token tiles, on the plan's bound
+    if (mid_deep(prob_n, n_deltas, prob_m, tile) && units32 <= 0x7fffffffL) {
+      a.tile_halves = tile == 64;
+      hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, true>), dim3((unsigned)units32), dim3(256), 0,
+                         static_cast<hipStream_t>(stream), a);
+      a.tile_halves = 0;
+    } else if (tile == 32)
       hipLaunchKernelGGL((sparse24_wide_kernel<1, 32, true>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
                          static_cast<hipStream_t>(stream), a);
     else
