@@ -245,7 +245,7 @@ def kernel_name(wl, lib, in_kernel):
         code = lib.triteia_hip_uniform_kernel(wl.m, groups, per_group, wl.k, 1)
         if code >= 1000:
             return f"sparse24_grouped_kernel (K split over {code - 1000} workgroups) + splitk_reduce_kernel"
-        return {0: "sparse24_grouped_kernel", 32: "sparse24_wide_kernel<32 tokens>", 33: "sparse24_wide_kernel<32 tokens, 8 wavefronts>",
+        return {0: "sparse24_grouped_kernel", 16: "sparse24_share16_kernel", 32: "sparse24_wide_kernel<32 tokens>", 33: "sparse24_wide_kernel<32 tokens, 8 wavefronts>",
                 64: "sparse24_wide_kernel<64 tokens>", 65: "sparse24_wide_kernel<64 tokens, 8 wavefronts>",
                 256: "sparse24_tile256_kernel"}.get(code, f"kernel code {code}")
     if in_kernel:
@@ -301,14 +301,32 @@ def measure(prob, wl, torch, ffi, steps, warmup, use_graph=True, reps=None):
     batch = 10
     reps = reps or max(3, min(20, steps // 10))
     durs = []
+    kgraph = None
+    if use_graph:
+        # the batch is replayed from a captured graph: launched one by one from Python, kernels shorter than the host's
+        # launch interval (about 9 us per call through ctypes) would be timed at that interval
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        kgraph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(kgraph, stream=side):
+                for i in range(batch):
+                    kernel_call(i)
+        torch.cuda.synchronize()
+        kgraph.replay()
+        torch.cuda.synchronize()
     for r in range(reps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for i in range(batch):
-            kernel_call(r * batch + i)
+        if kgraph is not None:
+            kgraph.replay()
+        else:
+            for i in range(batch):
+                kernel_call(r * batch + i)
         e1.record()
         e1.synchronize()
         durs.append(e0.elapsed_time(e1) / batch * 1e-3)
+    del kgraph
     kdur = float(np.median(durs))
     abytes = wl.delta_algorithmic_bytes()
     achieved = abytes / kdur / 1e9

@@ -98,7 +98,8 @@ TRITEIA_HIP_API int triteia_hip_bmm_2_4_tokens_scratch(const void* A, const void
 TRITEIA_HIP_API size_t triteia_hip_bmm_scratch_bytes(int prob_m, int batch, int tokens, int prob_k);
 
 /* Which kernel the uniform-group entry points (mul_2_4: batch = 1; bmm_2_4*) run most of a launch's rows on: 0 = the
- * K-split streaming kernel (sparse24_grouped_kernel), 1000 + n = the same with K split over n workgroups (only
+ * K-split streaming kernel (sparse24_grouped_kernel), 16 = shares of 16, 32 or 64 columns on sparse24_share16_kernel (at most 16 tokens per
+ * matrix, launches of at most 32 / 64 / 128 column blocks of 128), 1000 + n = the same with K split over n workgroups (only
  * with_scratch != 0), 32 / 64 = 32- / 64-token tiles of sparse24_wide_kernel (+ 1: on eight wavefronts), 256 =
  * sparse24_tile256_kernel; -1 for a shape the entry points reject.  No counterpart in the reference; for benchmarks,
  * profiles and the test that guards the dispatch thresholds. */

@@ -103,10 +103,13 @@ def test_dispatch_queries_at_the_documented_points():
     lib = _ffi.lib()
     _ffi.reload_env()
     uniform = lib.triteia_hip_uniform_kernel          # (m, batch, tokens, k, with_scratch)
-    assert uniform(4096, 1, 16, 4096, 1) == 0          # cfg0: K of 4096 is too short for a split across workgroups
+    assert uniform(4096, 1, 16, 4096, 1) == 16         # cfg0: K of 4096 is too short for a split across workgroups; 16-column shares
+    assert uniform(4096, 1, 17, 4096, 1) == 0          # more than one 16-token pass: the streaming kernel
+    assert uniform(11008, 1, 16, 4096, 1) == 16        # 86 column blocks: shares of 64 columns
+    assert uniform(28672, 1, 16, 4096, 1) == 0         # 224 column blocks: the streaming kernel
     assert uniform(4096, 8, 1, 4096, 1) == 0           # cfg1: a workgroup per CU already
     assert uniform(8192, 1, 16, 8192, 1) == 1004       # long K, few workgroups: K split in 4 ...
-    assert uniform(8192, 1, 16, 8192, 0) == 0          # ... only with a scratch buffer
+    assert uniform(8192, 1, 16, 8192, 0) == 16         # ... only with a scratch buffer (without: shares of 32 columns)
     assert lib.triteia_hip_bmm_scratch_bytes(8192, 1, 16, 8192) == 4 * 16 * 8192 * 4
     assert lib.triteia_hip_bmm_scratch_bytes(4096, 1, 16, 4096) == 0
     assert uniform(4096, 1, 1024, 4096, 1) == 33       # 32-token tiles on eight wavefronts (one workgroup per CU)

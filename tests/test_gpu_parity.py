@@ -115,7 +115,7 @@ def test_matmul_many_tokens_reference_test_shape(ops):
     (1, 1, 512, 256, 2, 41), (1, 16, 512, 384, 3, 42),  # forced splits; 3 does not divide the 4 steps
     (1, 40, 1024, 256, 4, 43), (1, 100, 448, 128, 2, 44),  # several token passes; a partial last step of K
     (1, 8, 192, 256, 5, 45),                            # more splits asked for than there are steps
-    (3, 5, 512, 256, 2, 46), (4, 1, 8192, 128, 0, 47),  # bmm, forced and by the rule
+    (3, 5, 512, 256, 2, 46), (4, 12, 8192, 128, 0, 47), # bmm, forced and by the rule
 ])
 def test_split_k_across_workgroups(ops, monkeypatch, b, n, k, m, ks, seed):
     """matmul / bmm launches of few workgroups split K across workgroups (fp32 partial sums in a scratch buffer, added
@@ -149,12 +149,21 @@ def test_split_k_across_workgroups(ops, monkeypatch, b, n, k, m, ks, seed):
     assert float((first.float() - unsplit.float()).norm() / unsplit.float().norm()) < 1e-4
 
 
-@pytest.mark.parametrize("b,n,k,m,seed", [(1, 16, 512, 384, 71), (1, 5, 4096, 256, 72), (3, 1, 1024, 128, 73), (2, 16, 192, 1152, 74)])
+@pytest.mark.parametrize("b,n,k,m,seed", [(1, 16, 512, 384, 71), (1, 5, 4096, 256, 72), (3, 1, 1024, 128, 73), (2, 16, 192, 1152, 74),
+                                          (1, 16, 11008, 256, 75),     # 86 steps: three chunks of requests per wavefront, the last ragged
+                                          (2, 7, 4096, 2048, 76),      # 32 column blocks in all: the most that take 16-column shares
+                                          (1, 3, 320, 128, 77),        # k = 320: a third step of two packed rows
+                                          (8, 1, 4096, 512, 78),       # one token on each of eight matrices
+                                          (1, 16, 1024, 5632, 79),     # 44 column blocks: shares of 32 columns
+                                          (3, 9, 768, 3584, 80),       # 84 column blocks: shares of 64 columns
+                                          (1, 2, 11008, 11008, 81)])   # 86 blocks, three chunks of requests
 def test_column_shares_keep_the_bits(ops, monkeypatch, b, n, k, m, seed):
     """Small matmul / bmm launches give a workgroup a share of a column block (64, 32 or 16 columns instead of 128).  Every
     output column is still summed by the same wavefronts in the same order: each share width gives the bits of the whole block,
-    and the oracle's values."""
+    and the oracle's values.  Left to the rule, these launches run on sparse24_share16_kernel (16-column shares, a share's
+    columns as the rows of the MFMA, all requests of a wavefront at once): the same bits again."""
     say(f"column shares b={b} n={n} k={k} m={m} seed={seed}")
+    from triteia_amd.python.capi import _ffi
     qw, meta, s = make_deltas(b, k, m, seed)
     x = activations(b * n, k, seed + 1).reshape(b, n, k)
     gq, gm, gs, gx = to_gpu(qw, meta, s, x)
@@ -170,10 +179,16 @@ def test_column_shares_keep_the_bits(ops, monkeypatch, b, n, k, m, seed):
     torch.cuda.synchronize()
     check_close(whole, ref, what="whole column blocks")
     for shift in (1, 2, 3):
+        if b * ((((m // 128) << shift) + 7) // 8 * 8) > 256:
+            continue        # (past one workgroup per CU the streaming kernel splits K over four wavefronts, not eight)
         setknob(monkeypatch, "TRITEIA_HIP_SUB_SHIFT", shift)
         assert torch.equal(call(), whole), f"shares of {128 >> shift} columns changed the result"
     delknob(monkeypatch, "TRITEIA_HIP_SUB_SHIFT")
-    assert torch.equal(call(), whole), "the rule's own choice of share changed the result"
+    assert _ffi.lib().triteia_hip_uniform_kernel(m, b, n, k, 0) == 16
+    assert torch.equal(call(), whole), "the rule's own choice (16-column shares on their own kernel) changed the result"
+    setknob(monkeypatch, "TRITEIA_HIP_SHARE16", 0)
+    assert _ffi.lib().triteia_hip_uniform_kernel(m, b, n, k, 0) == 0
+    assert torch.equal(call(), whole), "the streaming kernel's own choice of share changed the result"
 
 
 def test_reference_shaped_entry_points_directly(ops):

@@ -32,6 +32,9 @@ ROUTED_ALTERNATIVES = {
 UNIFORM_ALTERNATIVES = {
     "K-split kernel": {"TRITEIA_HIP_WIDE": "0", "TRITEIA_HIP_KSPLIT": "0"},
     "K split across workgroups": {"TRITEIA_HIP_WIDE": "0", "TRITEIA_HIP_KSPLIT": "4"},
+    "streaming kernel instead of column shares": {"TRITEIA_HIP_SHARE16": "0"},
+    "column shares instead of a K split": {"TRITEIA_HIP_KSPLIT": "0"},
+    "column shares on any launch of at most 16 tokens": {"TRITEIA_HIP_SHARE16_MAX_BLOCKS": BIG, "TRITEIA_HIP_KSPLIT": "0"},
     "whole column blocks": {"TRITEIA_HIP_SUB_SHIFT": "0"},
     "shares of 64 columns": {"TRITEIA_HIP_SUB_SHIFT": "1"},
     "32-token wide tiles": {"TRITEIA_HIP_TILE256": "0", "TRITEIA_HIP_KSPLIT": "0", "TRITEIA_HIP_WIDE32_MIN_UNITS": "1", "TRITEIA_HIP_WIDE32_MAX_UNITS": BIG, "TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS": "0", "TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS": "0"},
@@ -63,6 +66,7 @@ UNIFORM_GRID = [
     (4096, 4096, 16), (4096, 4096, 128), (4096, 4096, 512), (4096, 4096, 640), (4096, 4096, 1024), (4096, 4096, 1536),
     (4096, 4096, 2048), (4096, 4096, 4096), (4096, 11008, 256), (4096, 11008, 512), (4096, 11008, 2048),
     (11008, 4096, 16), (11008, 4096, 640), (11008, 4096, 2048), (8192, 8192, 16), (4096, 11008, 16),
+    (4096, 4096, 1), (4096, 8192, 16), (8192, 8192, 4), (14336, 4096, 4), (4096, 28672, 8),
 ]
 
 

@@ -14,6 +14,7 @@
 #include "probes.hip.h"
 #include "route_plan.hip.h"
 #include "sparse24_gemm.hip.h"
+#include "sparse24_share.hip.h"
 #include "sparse24_tile256.hip.h"
 #include "sparse24_wide.hip.h"
 
@@ -60,7 +61,7 @@ struct Knobs {
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
   int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
-  int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset;
+  int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset, share16 = 1, share16_max_blocks = kUnset;
 };
 Knobs g_knobs;
 std::once_flag g_knobs_once;
@@ -76,7 +77,7 @@ void read_knobs() {
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
       {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
       {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
-      {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift},
+      {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift}, {"SHARE16", &k.share16}, {"SHARE16_MAX_BLOCKS", &k.share16_max_blocks},
   };
   char name[64];
   for (auto& e : table) {
@@ -142,6 +143,19 @@ void launch_one(const Sparse24Args& a, dim3 grid, hipStream_t st) {
 
 // `nt`: token tile class; `tsplit`: workgroups along y sharing one group's tokens (run-table form
 // only: plan tiles never exceed one pass, uniform groups are cut into chunks by the kernel).
+// Decode-size uniform launches of at most 128 column blocks in all (a single matrix of up to 16384 columns): shares of
+// 16, 32 or 64 columns -- the narrowest that leaves at most one workgroup per CU -- on the kernel whose MFMA rows are
+// a share's columns and whose wavefronts request all their steps at once (sparse24_share.hip.h); same sums in the same
+// order as the eight-wavefront streaming kernel that took them before.  Returns the 16-column tiles per share, 0 = no.
+constexpr long kShare16MaxBlocks = 128;
+static int share16_tiles(long n_groups, int m, int tokens_per_group) {
+  if (tokens_per_group > 16 || !knobs().share16 || knobs().sub_shift != kUnset || knobs().kw != kUnset ||
+      knobs().depth != kUnset || knobs().nt != 0)
+    return 0;
+  const long blocks = n_groups * (m / 128);
+  if (blocks > knob_or(knobs().share16_max_blocks, kShare16MaxBlocks)) return 0;
+  return blocks <= 32 ? 1 : blocks <= 64 ? 2 : 4;
+}
 int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsplit = 1) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   if (tsplit < 1) tsplit = 1;
@@ -186,11 +200,21 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
   // About 512 workgroups run at a time.  When those belong to four or more deltas (narrow matrices),
   // the deltas start their walks over K spread evenly around the ring of steps; wide matrices are
   // streamed one or two at a time anyway and walk from step 0.
+  // (counted in whole column blocks, whatever the share a workgroup takes: the start of a delta's walk fixes the order
+  // of its fp32 sums, which must not depend on the share)
   {
-    const long side_by_side = 512 / cb_pad;
+    const long side_by_side = 512 / (((long)(a.m / 128) + 7) / 8 * 8);
     const int n_steps = (a.k / 32 + 3) / 4;
     const long spread = side_by_side >= 4 ? n_steps / (side_by_side < 16 ? side_by_side : 16) : 0;
     a.rot_spread = knob_or(knobs().rot_spread, spread);
+  }
+  if (const int tiles = uniform && nt == 1 && tsplit == 1 && zsplit == 1 && !a.ksplit_steps ? share16_tiles(a.n_groups, a.m, a.uniform_count) : 0) {
+    const long sh_pad = ((long)(a.m / (16 * tiles)) + 7) / 8 * 8;
+    const dim3 grid((unsigned)(a.n_groups * sh_pad));
+    if (tiles == 1) hipLaunchKernelGGL((sparse24_share16_kernel<8, 4, 1>), grid, dim3(512), 0, st, a);
+    else if (tiles == 2) hipLaunchKernelGGL((sparse24_share16_kernel<8, 4, 2>), grid, dim3(512), 0, st, a);
+    else hipLaunchKernelGGL((sparse24_share16_kernel<8, 4, 4>), grid, dim3(512), 0, st, a);
+    return check_launch("sparse24_share16_kernel");
   }
   const long units = (long)a.n_groups * cb_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
@@ -315,6 +339,7 @@ struct UniformPlan { UniformSegment seg[3]; int n = 0; };
 constexpr long kSplitKMaxUnits = 64;    // launches of at most this many unsplit workgroups are split ...
 constexpr int kSplitKMinSteps = 64;     // ... if K has at least this many steps of 128 ...
 constexpr int kSplitKStepsPerSplit = 16;   // ... into shares of about this many steps
+static int share16_tiles(long n_groups, int m, int tokens_per_group);
 int pick_ksplit(long tokens, long n_groups, int m, int k) {
   if (!knobs().ksplit || tokens <= 0) return 1;
   const long cb_pad = (m / 128 + 7) / 8 * 8;
@@ -323,6 +348,11 @@ int pick_ksplit(long tokens, long n_groups, int m, int k) {
   const int n_steps = (k / 32 + 3) / 4;
   if (knobs().ksplit > 1) return knobs().ksplit <= n_steps ? knobs().ksplit : n_steps;   // forced (tests, measurements)
   if (units > kSplitKMaxUnits || n_steps < kSplitKMinSteps) return 1;
+  // A handful of tokens: the column-share kernel (one launch, all of a wavefront's requests at once) is ahead of the
+  // split and its second launch as long as the activations that every share reads again are few (1 / 8 tokens on
+  // 8192 x 8192 11.4 / 12.7 against 13.4 / 13.9 us, on 11008 x 4096 10.4 / 13.5 against 13.3 / 14.0; 2 / 4 tokens on
+  // 14336 x 4096 13.3 / 15.2 against 13.9 / 14.2; 16 tokens on 11008 x 4096 16.8 against 14.6 us).
+  if (share16_tiles(n_groups, m, (int)tokens) && (tokens * (long)k <= 49152 || (k <= 11008 && tokens <= 8))) return 1;
   long ks = n_steps / kSplitKStepsPerSplit;
   if (ks > 512 / units) ks = 512 / units;
   if (ks > 16) ks = 16;
@@ -539,7 +569,7 @@ int triteia_hip_uniform_kernel(int prob_m, int batch, int tokens, int prob_k, in
   for (int i = 1; i < up.n; i++) if (up.seg[i].count > up.seg[best].count) best = i;
   const UniformSegment& sg = up.seg[best];
   if (sg.kind == kUniSplitK) return kUniSplitK + sg.ksplit;
-  if (sg.kind == kUniNarrow) return 0;
+  if (sg.kind == kUniNarrow) return share16_tiles(batch, prob_m, sg.count) ? 16 : 0;
   // 32- and 64-token tiles: + 1 when the launch runs on workgroups of eight wavefronts (halves of K)
   const long cgs = (prob_m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
   if (sg.kind == kUniWide32)
