@@ -249,6 +249,8 @@ def kernel_name(wl, lib, in_kernel):
                 64: "sparse24_wide_kernel<64 tokens>", 65: "sparse24_wide_kernel<64 tokens, 8 wavefronts>",
                 256: "sparse24_tile256_kernel"}.get(code, f"kernel code {code}")
     if in_kernel:
+        if lib.triteia_hip_routed_in_kernel(wl.tokens, wl.n_deltas, wl.m, wl.k) == 2:
+            return "sparse24_share16_kernel (routes in-kernel)"
         return "sparse24_grouped_kernel (routes in-kernel)"
     if wl.index_offset:
         return "sparse24_grouped_kernel"

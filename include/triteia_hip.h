@@ -193,8 +193,9 @@ TRITEIA_HIP_API int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas);
  * kernels add over K in different orders). */
 TRITEIA_HIP_API int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k);
 
-/* 1 if triteia_hip_sbmm_2_4_routed handles this batch and layer in one launch, routing inside the multiply kernel
- * (the workspace stays untouched), 0 if it builds a routing plan first.  No counterpart in the reference; for
+/* 1 or 2 if triteia_hip_sbmm_2_4_routed handles this batch and layer in one launch, routing inside the multiply kernel
+ * (the workspace stays untouched; 2: at most 16 tokens on the column-share kernel, sparse24_share16_kernel, 1: the
+ * streaming kernel), 0 if it builds a routing plan first.  No counterpart in the reference; for
  * benchmarks and profiles. */
 TRITEIA_HIP_API int triteia_hip_routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k);
 

@@ -126,6 +126,10 @@ def test_dispatch_queries_at_the_documented_points():
     assert routed(64, 32, 11008, 4096) == 0            # 33 .. 64 tokens over many deltas of a large layer: planned ...
     assert lib.triteia_hip_plan_tile_tokens(64, 32) == 32   # ... in 32-token tiles (a skewed batch's hot delta in one tile)
     assert routed(32, 32, 11008, 4096) == 1
+    assert routed(1, 16, 4096, 4096) == 2              # one token: column shares, routed in the kernel
+    assert routed(4, 16, 4096, 4096) == 2              # at most four deltas in use: 128 column blocks on the bound
+    assert routed(8, 16, 4096, 4096) == 1              # up to eight: the streaming kernel
+    assert routed(16, 4, 4096, 4096) == 1              # four tokens per delta: weights requested ahead of the routing
     assert routed(256, 32, 11008, 4096) == 0           # cfg3: planned ...
     assert lib.triteia_hip_planned_tile_kernel(256, 32, 11008, 4096) == 32   # ... and its 32-token tiles go to the wide kernel
     assert lib.triteia_hip_planned_tile_kernel(256, 16, 4096, 4096) == 0     # a narrow layer keeps the streaming kernel

@@ -420,6 +420,53 @@ def test_routing_is_bit_exact_on_exact_arithmetic(ops, monkeypatch, T, N, k, m, 
     assert torch.equal(ops.sbmm_4bit_2_4_multilaunch(gq, gxs, gm, gs, gis), wants)
 
 
+@pytest.mark.parametrize("T,N,k,m,seed", [
+    (1, 16, 4096, 512, 201),       # one token: one delta in use, 16-column shares
+    (3, 40, 1024, 1152, 202),      # three tokens over three of 40 deltas: 27 column blocks on the bound
+    (16, 4, 640, 2048, 203),       # 16 tokens over four deltas (requested ahead of the routing unless that is switched off)
+    (16, 64, 320, 1024, 204),      # up to 16 deltas in use of 64: 128 column blocks on the bound, shares of 64 columns; ragged K
+    (7, 5, 11008, 128, 205),       # a long K: three chunks of requests per wavefront
+    (5, 3, 256, 3584, 206),        # 84 column blocks on the bound
+])
+def test_small_routed_batches_on_column_shares(ops, monkeypatch, T, N, k, m, seed):
+    """A routed batch of at most 16 tokens over few deltas of a small layer runs on the column-share kernel (routing inside
+    the kernel, four wavefronts): against the oracle, the same bits as the streaming kernel, the same bits for a token
+    when its batch is larger, rows without a delta untouched, accumulation in place."""
+    say(f"small routed batch on column shares T={T} N={N} k={k} m={m} seed={seed}")
+    from triteia_amd.python.capi import sbmm_2_4_routed
+    setknob(monkeypatch, "TRITEIA_HIP_EAGER", "0")          # (route first: the form that takes the column-share kernel)
+    qw, meta, s = make_deltas(N, k, m, seed)
+    big = 48
+    x = activations(big, k, seed + 1)
+    rng = np.random.default_rng(seed + 2)
+    idx = rng.integers(-1, N, size=big).astype(np.int32)
+    idx[0] = N - 1                                           # (at least one routed token in the small batch)
+    if T >= 3:
+        idx[1] = -1
+    ref = orc.sbmm_4bit_2_4(qw, x, meta, s, idx)
+    gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
+
+    def run(n_tokens, accumulate=False, base=None):
+        out = torch.full((n_tokens, m), 3.0, dtype=torch.float16, device=DEV) if base is None else base.clone()
+        sbmm_2_4_routed(gx[:n_tokens], gq, gm, out, gs, gi[:n_tokens], accumulate=accumulate)
+        torch.cuda.synchronize()
+        return out
+
+    small = run(T)
+    none = torch.from_numpy(idx[:T] < 0).to(DEV)
+    assert bool((small[none] == 3.0).all())
+    check_close(torch.where(none[:, None], torch.zeros_like(small), small), ref[:T], what="column shares, routed")
+    setknob(monkeypatch, "TRITEIA_HIP_SHARE16", "0")
+    assert torch.equal(run(T), small), "the streaming kernel gives other bits"
+    delknob(monkeypatch, "TRITEIA_HIP_SHARE16")
+    whole = run(big)                                         # the same tokens inside a batch of 48
+    assert torch.equal(torch.where(none[:, None], whole[:T], whole[:T]), torch.where(none[:, None], whole[:T], small))
+    base = torch.from_numpy(activations(T, m, seed + 3)).to(DEV)
+    acc = run(T, accumulate=True, base=base)
+    assert torch.equal(acc[none], base[none])
+    check_close(acc.float() - base.float(), ref[:T], tol=4e-3, what="column shares, routed, accumulate")
+
+
 @pytest.mark.parametrize("T,N,used,seed", [
     (64, 16, [0, 3, 5, 15], 41),        # most deltas without tokens: their prefetched weights are dropped
     (64, 8, list(range(8)), 42),         # every delta in use, some with more than one 16-token pass

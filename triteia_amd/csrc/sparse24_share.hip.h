@@ -17,8 +17,11 @@
 
 namespace triteia_hip {
 
-// T: 16-column tiles of a share (1, 2 or 4)
-template <int KW, int DEPTH, int T>
+// T: 16-column tiles of a share (1, 2 or 4).  ROUTED: the groups are the deltas that a batch of at most 16 tokens uses,
+// worked out by every wavefront from the batch's indices (Sparse24Args::raw_indices), as sparse24_grouped_kernel does
+// for batches of up to 256; with KW = 4, the number of wavefronts that kernel keeps for routed tokens, so that a token's
+// bits do not depend on which of the two kernels its batch went to.
+template <int KW, int DEPTH, int T, bool ROUTED = false>
 __global__ __launch_bounds__(64 * KW, 2) void sparse24_share16_kernel(const Sparse24Args p) {
   constexpr int kShareCols = 16 * T;
   __shared__ float red[KW][16][kShareCols + 4];   // [wavefront][token][column of the share] (+ pad)
@@ -31,16 +34,40 @@ __global__ __launch_bounds__(64 * KW, 2) void sparse24_share16_kernel(const Spar
   const int i = unit - grp * sh_pad;
   const int sh = p.xcd_swizzle ? (i & 7) * (sh_pad >> 3) + (i >> 3) : i;
   if (sh >= shares || grp >= p.n_groups) return;
-  // uniform groups only: group g = delta g * delta_step with uniform_count (<= 16) rows
-  const int delta = grp * p.delta_step;
-  const int start = grp * p.uniform_stride + p.uniform_first;
-  const int cnt = min(p.uniform_count, 16);
-  if (delta < 0 || delta >= p.n_deltas || cnt <= 0) return;
-
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int rho = lane & 15;     // A: column rho of the share; B and D: token rho
   const int q = lane >> 4;       // A, B: packed row tr0 + q resp. k slots; D: columns 4q .. 4q + 3
+  int delta, start, cnt;
+  int list = 0;                  // ROUTED: lane s holds the batch position of the group's s-th token
+  if (ROUTED) {
+    // lane l < raw_count looks at token l; group g is the g-th delta in use, in ascending order
+    int d = p.raw_indices[min(lane, p.raw_count - 1)] - p.raw_offset;
+    if (lane >= p.raw_count || lane >= 16 || d < 0 || d >= p.n_deltas || d >= 64) d = -1;
+    unsigned long long used = d >= 0 ? (1ull << d) : 0ull;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const unsigned lo = __shfl_xor((unsigned)used, off, 64);
+      const unsigned hi = __shfl_xor((unsigned)(used >> 32), off, 64);
+      used |= ((unsigned long long)hi << 32) | lo;
+    }
+    if (grp >= __popcll(used)) return;
+    for (int g = 0; g < grp; g++) used &= used - 1;
+    delta = __ffsll((long long)used) - 1;
+    const unsigned long long members = __ballot(d == delta);
+    cnt = __popcll(members);
+    const int rank = __popcll(members & ((1ull << lane) - 1ull));
+    const int dest = (d == delta) ? rank : cnt + (lane - rank);   // a permutation: members first, in batch order
+    list = __builtin_amdgcn_ds_permute(dest << 2, lane);
+    start = 0;
+  } else {
+    // uniform groups: group g = delta g * delta_step with uniform_count (<= 16) rows
+    delta = grp * p.delta_step;
+    start = grp * p.uniform_stride + p.uniform_first;
+    cnt = min(p.uniform_count, 16);
+  }
+  if (delta < 0 || delta >= p.n_deltas || cnt <= 0) return;
+
   const int k_rows = p.k >> 5;
   const int n_steps = (k_rows + 3) >> 2;
   const int rot = (int)(((unsigned)delta * (unsigned)p.rot_spread) % (unsigned)n_steps);
@@ -61,7 +88,7 @@ __global__ __launch_bounds__(64 * KW, 2) void sparse24_share16_kernel(const Spar
   const int w_shift = (c >> 2) * 8;
   const int m_shift = (c >> 2) * 16;
   // B operand: token slot rho (slots past the end repeat the last row; their results are dropped)
-  const long row = start + min(rho, cnt - 1);
+  const long row = ROUTED ? __shfl(list, min(rho, cnt - 1), 64) : start + min(rho, cnt - 1);
   const _Float16* xrow = p.x + row * p.x_stride + 32 * (q >> 1) + 8 * (q & 1);
 
   struct Frag {
@@ -140,6 +167,8 @@ __global__ __launch_bounds__(64 * KW, 2) void sparse24_share16_kernel(const Spar
 #pragma unroll
   for (int t = 0; t < T; t++) *reinterpret_cast<float4_t*>(&red[wave][rho][16 * t + 4 * q]) = acc[t];
   __syncthreads();
+  // (the row of a routed token is fetched from the lane that holds it while every lane is active)
+  const long orow_routed = ROUTED ? __shfl(list, (tid / (2 * T)) & 15, 64) : 0;
   if (tid < 32 * T) {
     const int tok = tid / (2 * T), f0 = (tid % (2 * T)) * 8;
     if (tok < cnt) {
@@ -154,7 +183,8 @@ __global__ __launch_bounds__(64 * KW, 2) void sparse24_share16_kernel(const Spar
         for (int e = 0; e < 4; e++) { v[e] += a0[e]; v[4 + e] += a1[e]; }
       }
       const half8_t sv = *reinterpret_cast<const half8_t*>(p.scales + (long)delta * p.scales_stride + sh * kShareCols + f0);
-      _Float16* op = p.out + (long)(start + tok) * p.out_stride + sh * kShareCols + f0;
+      const long orow = ROUTED ? orow_routed : start + tok;
+      _Float16* op = p.out + orow * p.out_stride + sh * kShareCols + f0;
       half8_t old = {0, 0, 0, 0, 0, 0, 0, 0};
       if (p.accumulate) old = *reinterpret_cast<const half8_t*>(op);
       half8_t o;

@@ -216,6 +216,16 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
     else hipLaunchKernelGGL((sparse24_share16_kernel<8, 4, 4>), grid, dim3(512), 0, st, a);
     return check_launch("sparse24_share16_kernel");
   }
+  // The same for a routed batch of at most 16 tokens that is routed inside the kernel (one group per delta in use, at
+  // most min(tokens, deltas) of them): on four wavefronts, like every routed launch.
+  if (const int tiles = a.raw_indices && !a.raw_static && nt == 1 && tsplit == 1 && zsplit == 1 ? share16_tiles(a.n_groups, a.m, a.raw_count) : 0) {
+    const long sh_pad = ((long)(a.m / (16 * tiles)) + 7) / 8 * 8;
+    const dim3 grid((unsigned)(a.n_groups * sh_pad));
+    if (tiles == 1) hipLaunchKernelGGL((sparse24_share16_kernel<4, 8, 1, true>), grid, dim3(256), 0, st, a);
+    else if (tiles == 2) hipLaunchKernelGGL((sparse24_share16_kernel<4, 4, 2, true>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((sparse24_share16_kernel<4, 4, 4, true>), grid, dim3(256), 0, st, a);
+    return check_launch("sparse24_share16_kernel (routed)");
+  }
   const long units = (long)a.n_groups * cb_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   const dim3 grid((unsigned)units, (unsigned)tsplit, (unsigned)zsplit);
@@ -793,7 +803,11 @@ int triteia_hip_probe_stream(const void* A, const void* B, const void* meta, voi
 
 int triteia_hip_routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
-  return routed_in_kernel(prob_n, n_deltas, prob_m, prob_k) ? 1 : 0;
+  if (!routed_in_kernel(prob_n, n_deltas, prob_m, prob_k)) return 0;
+  // (the launch that sbmm_2_4_routed makes of it: route first unless there are two tokens per delta; 16-token passes)
+  const bool shares = prob_n <= 16 && !routed_eager_ok(prob_n, n_deltas) && pick_nt(prob_n, prob_n < n_deltas ? prob_n : n_deltas) == 1 &&
+                      share16_tiles(prob_n < n_deltas ? prob_n : n_deltas, prob_m, prob_n);
+  return shares ? 2 : 1;
 }
 
 int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
