@@ -78,18 +78,30 @@ def set_env(env):
 
 
 def time_call(call, reps=15, batch=10):
+    """Microseconds per call: `batch` calls captured in a graph and replayed between two events, `reps` times (launched
+    one by one from Python, kernels shorter than the host's launch interval would all measure the same)."""
     for i in range(3):
         call(i)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(batch):
+                call(i)
+    torch.cuda.synchronize()
+    graph.replay()
     torch.cuda.synchronize()
     times = []
     for r in range(reps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for i in range(batch):
-            call(r * batch + i)
+        graph.replay()
         e1.record()
         e1.synchronize()
         times.append(e0.elapsed_time(e1) / batch * 1e3)
+    del graph
     return float(np.median(times))
 
 
@@ -156,10 +168,9 @@ def test_default_rule_against_forced_alternatives_routed():
         ws = torch.empty((nbytes + 3) // 4, dtype=torch.int32, device=DEV)
 
         def make_call():
-            stream = _ffi.stream_of(x)
-
             def call(i):
                 q, me, s = weights[i % len(weights)]
+                stream = _ffi.stream_of(x)              # (torch's current stream: the capturing one while a graph is recorded)
                 rc = lib.triteia_hip_sbmm_2_4_routed(P(x), P(q), P(me), P(out), P(s), P(idx), 0, n, m, t, k, P(ws), ws.numel() * 4, 0, 0, stream)
                 assert rc == 0, _ffi.last_error()
             return call
@@ -189,10 +200,9 @@ def test_default_rule_against_forced_alternatives_uniform():
         scratch = torch.empty(64 << 20, dtype=torch.uint8, device=DEV)
 
         def make_call():
-            stream = _ffi.stream_of(x)
-
             def call(i):
                 q, me, s = weights[i % len(weights)]
+                stream = _ffi.stream_of(x)
                 rc = lib.triteia_hip_bmm_2_4_tokens_scratch(P(x), P(q), P(me), P(out), P(s), m, 1, t, k, P(scratch), scratch.numel(), 0, stream)
                 assert rc == 0, _ffi.last_error()
             return call
