@@ -67,7 +67,7 @@ def test_other_argument_errors():
     assert lib.triteia_hip_planned_tile_kernel(256, 32, 11008, 4096) == 32      # cfg3: wide layer, 32-token tiles
     assert lib.triteia_hip_planned_tile_kernel(256, 16, 4096, 4096) == 0        # narrow layer: the K-split kernel
     assert lib.triteia_hip_planned_tile_kernel(2048, 32, 11008, 4096) == 64
-    assert lib.triteia_hip_planned_tile_kernel(2048, 64, 28672, 8192) == 0      # 64-token tiles, long K
+    assert lib.triteia_hip_planned_tile_kernel(2048, 64, 28672, 8192) == 64     # 64-token tiles on a long K as well
     one = ctypes.c_void_p(16)
     assert lib.triteia_hip_route_plan(one, 0, 16, 64, one, need - 1, 0, null) == _ffi.ERR_ARGUMENT
     assert lib.triteia_hip_route_plan(one, 0, 100000, 64, one, 1 << 30, 0, null) == _ffi.ERR_KERN_SHAPE

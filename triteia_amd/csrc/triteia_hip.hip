@@ -59,7 +59,7 @@ struct Knobs {
   int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
-  int mid = 1, mid64 = 1, mid64_max_k = 8192, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0;
+  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
   int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset, share16 = 1, share16_max_blocks = kUnset;
 };
@@ -688,8 +688,10 @@ static bool mid_deep(int prob_n, int n_deltas, int prob_m, int tile) {
 }
 static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   const int tile = triteia_hip_plan_tile_tokens(prob_n, n_deltas);
-  // (64-token plans as well, on the 64-token build, where K is short: cfg3 at 1024 / 2048 tokens 196 -> 170 /
-  // 250 -> 214 us; at k = 8192 the narrow kernel's workgroups live long enough: cfg4 at 2048 tokens 1478 -> 1523 us)
+  // (64-token plans as well, on the 64-token build: cfg3 at 1024 / 2048 tokens 196 -> 170 / 250 -> 214 us; 8192 x 28672
+  // with 2048 / 4096 tokens over 64 deltas 1454 -> 1317 / 1920 -> 1736 us, 2048 tokens over 32 deltas 985 -> 864 us;
+  // 8192 x 8192 with 4096 tokens over 64 deltas 408 -> 381 us; k = 11008 .. 28672: 0-3 % faster.  The knob mid64_max_k
+  // can cap it: before the wide kernel's loop lost its conditional waits, k >= 8192 was better off on the narrow kernel.)
   const bool mid64 = tile == 64 && knobs().mid64 && prob_k < knobs().mid64_max_k;
   if (!knobs().mid || (tile != 32 && !mid64)) return false;
   if (prob_k % 128 != 0 || (long)prob_n * prob_k * 2 >= (1L << 32)) return false;   // whole K steps, 32-bit activation offsets
