@@ -165,7 +165,7 @@ TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_static_max_bytes(void);
 
 /* Only the routing step of triteia_hip_sbmm_2_4_routed: fills `workspace` (16-byte aligned) with
  *   int32 header[8] = {narrow tiles, routed tokens, deltas in use, narrow tile size,
- *                      wide tiles, tiles of all[], 0, 0}
+ *                      wide tiles, tiles of all[], tiles of big[], 0}
  *   int32 tiles[max_tiles][4] = {delta, start, count, 0}: at most `tile size` tokens of one
  *         delta, listed at perm[start .. start+count); a delta's tiles are adjacent
  *   int32 wide[max_wide][4]   = the same for 64-token tiles; only batches of at least 256
@@ -178,7 +178,11 @@ TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_static_max_bytes(void);
  *         {tiles, wide} or {all} per weight shape on the device: the wide kernel runs only if
  *         its tiles fill the chip (wide tiles x ceil(prob_m / 512) >= 150, environment
  *         TRITEIA_HIP_PLAN_WIDE_MIN_UNITS); the LoRA path always takes all[].
- * with max_tiles = min(prob_n, n_deltas) + prob_n / 16 and max_wide = prob_n / 33 + 1.  The
+ *   int32 big[max_big][4]     = for batches of at least 48 tokens per delta (of min(prob_n, n_deltas) deltas) whose
+ *         narrow tile size is 32: the same tokens cut into 64-token tiles only (header[6] of them), which wide layers
+ *         take on the 64-token build of the wide kernel (environment TRITEIA_HIP_PLAN_BIG=0: never)
+ * with max_tiles = min(prob_n, n_deltas) + prob_n / 16, max_wide = prob_n / 33 + 1 and
+ * max_big = min(prob_n, n_deltas) + prob_n / 64.  The
  * narrow tile size is triteia_hip_plan_tile_tokens(prob_n, n_deltas).  Exposed so that one
  * routing pass can serve every layer of a forward pass and the LoRA path. */
 TRITEIA_HIP_API int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_deltas, int prob_n, void* workspace,
@@ -188,7 +192,8 @@ TRITEIA_HIP_API int triteia_hip_plan_tile_tokens(int prob_n, int n_deltas);
 
 /* Which kernel triteia_hip_sbmm_2_4_planned runs a plan's narrow tiles on for this batch and layer:
  * 0 = the K-split narrow kernel (sparse24_grouped_kernel), 32 / 64 = the 32- / 64-token build of the
- * wide kernel taking the plan's narrow-only list (wide layers; see the design notes).  No counterpart in
+ * wide kernel taking the plan's narrow-only list, or its list of 64-token tiles where the narrow tiles are of 32
+ * (wide layers; see the design notes).  No counterpart in
  * the reference; for benchmarks and profiles, and for tests that compare results bit for bit (the two
  * kernels add over K in different orders). */
 TRITEIA_HIP_API int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k);

@@ -59,7 +59,7 @@ def test_other_argument_errors():
     assert lib.triteia_hip_bgmv(null, null, null, null, 4, 4096, 16, 1, 3, 1.0, 0, null) == _ffi.ERR_PROB_SHAPE
     # routed sbmm: workspace too small, too many deltas
     need = lib.triteia_hip_sbmm_routed_workspace_bytes(64, 16)
-    assert need == 4 * (8 + 4 * (16 + 64 // 16) + 4 * (64 // 33 + 1) + 64 + 4 * (16 + 64 // 16))
+    assert need == 4 * (8 + 4 * (16 + 64 // 16) + 4 * (64 // 33 + 1) + 64 + 4 * (16 + 64 // 16) + 4 * (16 + 64 // 64))
     assert lib.triteia_hip_plan_tile_tokens(8, 8) == 16
     assert lib.triteia_hip_plan_tile_tokens(64, 16) == 16       # at most 4 tokens per delta on average
     assert lib.triteia_hip_plan_tile_tokens(256, 16) == 32
@@ -68,6 +68,11 @@ def test_other_argument_errors():
     assert lib.triteia_hip_planned_tile_kernel(256, 16, 4096, 4096) == 0        # narrow layer: the K-split kernel
     assert lib.triteia_hip_planned_tile_kernel(2048, 32, 11008, 4096) == 64
     assert lib.triteia_hip_planned_tile_kernel(2048, 64, 28672, 8192) == 64     # 64-token tiles on a long K as well
+    # 1024 tokens over 8 deltas: the plan is cut in 32-token tiles and lists 64-token tiles beside them for wide layers
+    assert lib.triteia_hip_plan_tile_tokens(1024, 8) == 32
+    assert lib.triteia_hip_planned_tile_kernel(1024, 8, 11008, 4096) == 64
+    assert lib.triteia_hip_planned_tile_kernel(1024, 8, 4096, 4096) == 32
+    assert lib.triteia_hip_planned_tile_kernel(1024, 32, 11008, 4096) == 32     # 32 tokens per delta: no 64-token tiles
     one = ctypes.c_void_p(16)
     assert lib.triteia_hip_route_plan(one, 0, 16, 64, one, need - 1, 0, null) == _ffi.ERR_ARGUMENT
     assert lib.triteia_hip_route_plan(one, 0, 100000, 64, one, 1 << 30, 0, null) == _ffi.ERR_KERN_SHAPE

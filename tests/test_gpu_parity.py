@@ -640,6 +640,50 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     check_close(acc.float() - base.float(), ref, tol=4e-3, what="32-token wide kernel, accumulate")
 
 
+@pytest.mark.parametrize("T,N,k,m,seed,counts", [
+    (2000, 10, 640, 384, 111, None),                        # past two workgroups per CU on the bound as it is
+    (700, 6, 256, 640, 112, None),                          # smaller: the two-deep build switched off
+    (640, 5, 384, 256, 113, (0, 64, 65, 31, 480)),          # no token, a full tile, one over, half a tile, many tiles
+    (1024, 16, 128, 128, 114, (64,) * 16),                  # every tile full, one K step, one column block
+])
+def test_plan_lists_64_token_tiles_for_wide_layers(ops, monkeypatch, T, N, k, m, seed, counts):
+    """A batch of 48 tokens per delta and more whose plan is cut in 32-token tiles also lists its tokens in 64-token
+    tiles, which wide layers run on the 64-token build of the wide kernel (forced here onto small layers).  Against
+    the oracle within the bar; the same bits as from the 32-token tiles; untouched rows stay untouched."""
+    say(f"64-token tiles beside a 32-token plan T={T} N={N} k={k} m={m} seed={seed}")
+    from triteia_amd.python.capi import sbmm_2_4_routed, _ffi
+    lib = _ffi.lib()
+    qw, meta, s = make_deltas(N, k, m, seed)
+    x = activations(T, k, seed + 1)
+    rng = np.random.default_rng(seed + 2)
+    if counts is None:
+        idx = rng.integers(-1, N, size=T).astype(np.int32)
+    else:
+        idx = np.concatenate([np.full(c, d, np.int32) for d, c in enumerate(counts)])
+        idx = rng.permutation(idx).astype(np.int32)
+        assert idx.size == T
+    ref = orc.sbmm_4bit_2_4(qw, x, meta, s, idx)
+    gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
+    outs = {}
+    for big in ("1", "0"):
+        setknob(monkeypatch, "TRITEIA_HIP_FUSED_ROUTE", "0")
+        setknob(monkeypatch, "TRITEIA_HIP_MID_MIN_UNITS", "1")
+        setknob(monkeypatch, "TRITEIA_HIP_MID_MIN_COLUMN_GROUPS", "1")
+        setknob(monkeypatch, "TRITEIA_HIP_MID_NARROW", "0")
+        setknob(monkeypatch, "TRITEIA_HIP_MID_DEPTH", "1")
+        setknob(monkeypatch, "TRITEIA_HIP_PLAN_BIG", big)
+        assert lib.triteia_hip_plan_tile_tokens(T, N) == 32
+        assert lib.triteia_hip_planned_tile_kernel(T, N, m, k) == (64 if big == "1" else 32)
+        out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
+        sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
+        torch.cuda.synchronize()
+        outs[big] = out
+    none = torch.from_numpy(idx < 0).to(DEV)
+    assert bool((outs["1"][none] == -3.0).all())
+    check_close(torch.where(none[:, None], torch.zeros_like(outs["1"]), outs["1"]), ref, what="64-token tiles beside a 32-token plan")
+    assert torch.equal(outs["1"], outs["0"]), "the 64-token tiles changed bits"
+
+
 def test_empty_and_degenerate_inputs(ops):
     """Zero tokens, zero deltas, zero adapters, a batch in which nothing is routed: every op returns the
     shape it should and touches nothing else."""

@@ -9,7 +9,8 @@
 // Output (all int32, in the caller's workspace):
 //   header[0] = number of narrow tiles, header[1] = number of routed tokens,
 //   header[2] = number of deltas that have at least one token, header[3] = narrow tile size,
-//   header[4] = number of wide tiles, header[5] = number of tiles in all[], header[6..7] = 0
+//   header[4] = number of wide tiles, header[5] = number of tiles in all[], header[6] = number of tiles in big[],
+//   header[7] = 0
 //   tiles[..] = {delta, start, count, 0}: `count` <= tile size tokens of one delta,
 //               listed at perm[start .. start+count); ascending delta id, a delta's
 //               tiles are adjacent
@@ -20,6 +21,8 @@
 //               delta (stable)
 //   all[..]   = (only with wide = 1) the same tokens cut into narrow tiles only: the consumer
 //               chooses between {tiles, wide} and {all} per weight shape, on the device
+//   big[..]   = (only when built with big = 1) the same tokens cut into 64-token tiles only, for the layers on which
+//               the consumer prefers those to the narrow tiles the plan was cut in
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -35,8 +38,8 @@ constexpr int kPlanCachedTokens = 8192;  // token indices kept in LDS between th
 constexpr int kPlanMinTile = 16;      // smallest tile size a plan can be built for
 
 struct PlanLayout {
-  int header, tiles, wide, perm, all, total;  // offsets in ints
-  int max_tiles, max_wide;
+  int header, tiles, wide, perm, all, big, total;  // offsets in ints
+  int max_tiles, max_wide, max_big;
 };
 
 // The layout depends only on (tokens, deltas), not on the tile size the plan is built
@@ -51,7 +54,9 @@ __host__ __device__ inline PlanLayout plan_layout(int n_tokens, int n_deltas) {
   l.wide = l.tiles + 4 * l.max_tiles;
   l.perm = l.wide + 4 * l.max_wide;
   l.all = (l.perm + n_tokens + 3) & ~3;
-  l.total = l.all + 4 * l.max_tiles;
+  l.big = l.all + 4 * l.max_tiles;
+  l.max_big = g + n_tokens / kPlanWideTile;
+  l.total = l.big + 4 * l.max_big;
   return l;
 }
 
@@ -79,7 +84,7 @@ __device__ __forceinline__ int wave_excl_scan(int v, int lane, int* total) {
 // that the wavefronts can place their shares side by side and the order inside a delta is still the batch's.
 __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __restrict__ indices, int n_tokens,
                                                                  int n_deltas, int index_offset, int tile, int wide,
-                                                                 int* __restrict__ ws) {
+                                                                 int big, int* __restrict__ ws) {
   __shared__ int s_cursor[kPlanMaxDeltas];     // [share][delta]: counts, then cursors into perm
   __shared__ int s_delta[kPlanCachedTokens];   // pass 1 leaves each token's delta here for pass 2
   const PlanLayout L = plan_layout(n_tokens, n_deltas);
@@ -106,10 +111,11 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
   if (wave == 0) {
     // exclusive scans over the deltas, 64 per iteration: token counts -> first slot in perm,
     // tile counts -> first tile
-    int running = 0, tiles = 0, wides = 0, alls = 0, groups = 0;
+    int running = 0, tiles = 0, wides = 0, alls = 0, bigs = 0, groups = 0;
     int4* tile_out = reinterpret_cast<int4*>(ws + L.tiles);
     int4* wide_out = reinterpret_cast<int4*>(ws + L.wide);
     int4* all_out = reinterpret_cast<int4*>(ws + L.all);
+    int4* big_out = reinterpret_cast<int4*>(ws + L.big);
     for (int base = 0; base < n_deltas; base += 64) {
       const int d = base + lane;
       int c = 0;
@@ -145,6 +151,16 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
         }
         alls += chunk_alls;
       }
+      if (big) {
+        int chunk_bigs;
+        const int nb = (c + kPlanWideTile - 1) / kPlanWideTile;
+        const int bpos = bigs + wave_excl_scan(nb, lane, &chunk_bigs);
+        for (int i = 0; i < nb; i++) {
+          const int first = i * kPlanWideTile;
+          big_out[bpos + i] = make_int4(d, offs + first, min(kPlanWideTile, c - first), 0);
+        }
+        bigs += chunk_bigs;
+      }
       if (d < n_deltas) {
         // the shares' pieces of this delta's run of slots, in the order of the shares
         int before = 0;
@@ -166,7 +182,7 @@ __global__ __launch_bounds__(kPlanThreads) void route_plan_kernel(const int* __r
       ws[L.header + 3] = tile;
       ws[L.header + 4] = wides;
       ws[L.header + 5] = alls;
-      ws[L.header + 6] = 0;
+      ws[L.header + 6] = bigs;
       ws[L.header + 7] = 0;
     }
   }

@@ -59,7 +59,7 @@ struct Knobs {
   int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
-  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0;
+  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
   int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset, share16 = 1, share16_max_blocks = kUnset;
 };
@@ -75,7 +75,7 @@ void read_knobs() {
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
       {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
-      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
+      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"PLAN_BIG", &k.plan_big}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
       {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
       {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift}, {"SHARE16", &k.share16}, {"SHARE16_MAX_BLOCKS", &k.share16_max_blocks},
   };
@@ -743,8 +743,27 @@ static int plan_has_wide(int prob_n, int n_deltas) {
   return wide_enabled() && prob_n >= knobs().wide_min_batch && prob_n >= 8 * groups;
 }
 
+// A batch of 48 tokens per delta and more that pick_nt cuts in 32-token tiles, because it has few tiles in all and
+// narrow layers then get twice the workgroups: its plan also lists the tokens in 64-token tiles, and a layer of 16
+// column groups and more whose plan tiles go to the wide kernel, in a launch past two workgroups per CU, takes
+// those on the 64-token build.  Measured (32-token tiles -> 64-token tiles, evenly routed): 4096 x 11008 with
+// 768 / 1024 / 2048 tokens over 8 deltas 78.5 -> 68.9, 86.9 -> 78.5, 156.8 -> 129.3 us; 8192 x 8192 with 1536 / 2048
+// over 8 deltas 159.6 -> 141.3, 210.7 -> 161.3 us; 8192 x 28672 with 512 / 1024 tokens over 8 deltas 232.9 -> 179.9,
+// 370.9 -> 319.3 us, with 1024 Zipf(1.2)-routed tokens over 8 / 16 deltas 398.6 -> 334.2, 493.7 -> 459.0 us.  With 32 tokens
+// per delta, where every second half of a 64-token tile is empty, it loses (4096 x 11008 with 1024 tokens over 32
+// deltas 122.9 -> 136.8 us), and narrow layers are better off with the workgroups of 32-token tiles.
+constexpr int kPlanBigMinTokensPerDelta = 48;
+static int plan_has_big(int prob_n, int n_deltas) {
+  const long groups = n_deltas < prob_n ? n_deltas : prob_n;
+  return knobs().plan_big && prob_n >= kPlanBigMinTokensPerDelta * groups && triteia_hip_plan_tile_tokens(prob_n, n_deltas) == 32;
+}
+static bool mid_big(int prob_n, int n_deltas, int prob_m, int prob_k) {
+  return plan_has_big(prob_n, n_deltas) && (prob_m / 128 + 3) / 4 >= knobs().mid_min_column_groups &&
+         mid_tiles(prob_n, n_deltas, prob_m, prob_k) && !mid_deep(prob_n, n_deltas, prob_m, 32);
+}
 int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
+  if (mid_big(prob_n, n_deltas, prob_m, prob_k)) return 64;
   return mid_tiles(prob_n, n_deltas, prob_m, prob_k) ? triteia_hip_plan_tile_tokens(prob_n, n_deltas) : 0;
 }
 
@@ -827,7 +846,8 @@ int triteia_hip_route_plan(const void* token_indices, int index_offset, int n_de
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   hipLaunchKernelGGL(route_plan_kernel, dim3(1), dim3(kPlanThreads), 0, static_cast<hipStream_t>(stream),
                      static_cast<const int*>(token_indices), prob_n, n_deltas, index_offset,
-                     triteia_hip_plan_tile_tokens(prob_n, n_deltas), plan_has_wide(prob_n, n_deltas), static_cast<int*>(workspace));
+                     triteia_hip_plan_tile_tokens(prob_n, n_deltas), plan_has_wide(prob_n, n_deltas), plan_has_big(prob_n, n_deltas),
+                     static_cast<int*>(workspace));
   return check_launch("route_plan_kernel");
 }
 
@@ -882,7 +902,18 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     const int forced = knobs().pass_nt;
     if ((forced == 1 || forced == 2 || forced == 4) && 16 * forced <= tile) pass_nt = forced;
   }
-  if (mid) {
+  if (mid && mid_big(prob_n, n_deltas, prob_m, prob_k)) {
+    // the plan's own list of 64-token tiles, whole, on the 64-token build
+    const long cgs = (a.m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
+    a.tiles = reinterpret_cast<const int4*>(ws + L.big);
+    a.tiles_alt = nullptr;
+    a.n_groups_dev = ws + L.header + 6;
+    a.n_groups = L.max_big;
+    if ((long)a.n_groups * cg_pad > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units");
+    hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), a);
+    if (int e = check_launch("sparse24_wide_kernel (plan tiles)")) return e;
+  } else if (mid) {
     const long cgs = (a.m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
     if ((long)a.n_groups * cg_pad > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units");
     const long units32 = (long)a.n_groups * (tile == 64 ? 2 : 1) * cg_pad;   // in 32-token tiles, on the plan's bound
