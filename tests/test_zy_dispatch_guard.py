@@ -24,8 +24,8 @@ ROUTED_ALTERNATIVES = {
     "plan, K-split kernel, 32-token tiles": {"TRITEIA_HIP_FUSED_ROUTE": "0", "TRITEIA_HIP_MID": "0", "TRITEIA_HIP_NT": "2", "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS": BIG},
     "plan, K-split kernel, 64-token tiles": {"TRITEIA_HIP_FUSED_ROUTE": "0", "TRITEIA_HIP_MID": "0", "TRITEIA_HIP_NT": "4", "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS": BIG},
     "plan, hot deltas on 64-token wide tiles": {"TRITEIA_HIP_FUSED_ROUTE": "0", "TRITEIA_HIP_MID": "0", "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS": "1"},
-    "plan, 32-token tiles on the wide kernel": {"TRITEIA_HIP_FUSED_ROUTE": "0", "TRITEIA_HIP_NT": "2", "TRITEIA_HIP_MID_MIN_UNITS": "1", "TRITEIA_HIP_MID_MIN_COLUMN_GROUPS": "1", "TRITEIA_HIP_MID_MIN_HALF_TOKENS": "0", "TRITEIA_HIP_MID_DEPTH": "1"},
-    "plan, 32-token tiles on the wide kernel, two steps in flight": {"TRITEIA_HIP_FUSED_ROUTE": "0", "TRITEIA_HIP_NT": "2", "TRITEIA_HIP_MID_MIN_UNITS": "1", "TRITEIA_HIP_MID_MIN_COLUMN_GROUPS": "1", "TRITEIA_HIP_MID_MIN_HALF_TOKENS": "0", "TRITEIA_HIP_MID_DEPTH": "2"},
+    "plan, 32-token tiles on the wide kernel": {"TRITEIA_HIP_FUSED_ROUTE": "0", "TRITEIA_HIP_NT": "2", "TRITEIA_HIP_MID_MIN_UNITS": "1", "TRITEIA_HIP_MID_MIN_COLUMN_GROUPS": "1", "TRITEIA_HIP_MID_MIN_HALF_TOKENS": "0", "TRITEIA_HIP_MID_DEPTH": "1", "TRITEIA_HIP_PLAN_BIG": "0"},
+    "plan, 32-token tiles on the wide kernel, two steps in flight": {"TRITEIA_HIP_FUSED_ROUTE": "0", "TRITEIA_HIP_NT": "2", "TRITEIA_HIP_MID_MIN_UNITS": "1", "TRITEIA_HIP_MID_MIN_COLUMN_GROUPS": "1", "TRITEIA_HIP_MID_MIN_HALF_TOKENS": "0", "TRITEIA_HIP_MID_DEPTH": "2", "TRITEIA_HIP_PLAN_BIG": "0"},
     "plan, 64-token tiles on the wide kernel": {"TRITEIA_HIP_FUSED_ROUTE": "0", "TRITEIA_HIP_NT": "4", "TRITEIA_HIP_MID_MIN_UNITS": "1", "TRITEIA_HIP_MID_MIN_COLUMN_GROUPS": "1", "TRITEIA_HIP_MID64_MAX_K": BIG, "TRITEIA_HIP_MID_MIN_HALF_TOKENS": "0", "TRITEIA_HIP_MID_DEPTH": "1"},
 }
 # ... and for a single-matrix product
@@ -55,12 +55,17 @@ ROUTED_GRID = [
     (4096, 11008, 32, 2048), (4096, 11008, 8, 256), (4096, 11008, 8, 1024),
     (11008, 4096, 32, 64), (11008, 4096, 32, 256), (11008, 4096, 32, 1024), (11008, 4096, 8, 512),
     (4096, 4096, 16, 768), (4096, 11008, 4, 512), (4096, 11008, 8, 768), (8192, 8192, 8, 512), (8192, 8192, 8, 1536),
+    (4096, 14336, 8, 1024), (4096, 14336, 16, 768), (8192, 8192, 16, 2048), (8192, 28672, 8, 512),
 ]
 # Points where the host cannot know which alternative is ahead, with the tolerance allowed there.  The two-deep build of the
 # wide kernel holds two workgroups per CU, the one-deep build three; past the point where the plan's upper bound of tiles
 # fits two per CU, which of them packs the batch's real number of (tile, column group) units into fewer rounds of
 # workgroups depends on the routing (here 858 units: 1.12 rounds of 768 against 1.68 of 512), and only the device has it.
-KNOWN_GAPS = {(4096, 11008, 32, 512): 1.15}
+# The other point: 2048 randomly routed tokens over 16 deltas leave 128 +- 11 per delta, so about half of the deltas spill a
+# few tokens into a third 64-token tile that costs a whole pass over the delta's weights (some 40 tiles x 16 column groups
+# = 640 workgroups, a quarter past the 512 that run together); the split into full 64-token tiles for the wide kernel and
+# rests for the K-split kernel keeps that launch within 512.  Whether a batch spills is again known on the device only.
+KNOWN_GAPS = {(4096, 11008, 32, 512): 1.15, (8192, 8192, 16, 2048): 1.15}
 # (k, m, tokens): single-matrix products around the windows of the wide kernels and of the K split
 UNIFORM_GRID = [
     (4096, 4096, 16), (4096, 4096, 128), (4096, 4096, 512), (4096, 4096, 640), (4096, 4096, 1024), (4096, 4096, 1536),

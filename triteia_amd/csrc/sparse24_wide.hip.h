@@ -48,19 +48,28 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
 
   // unit = (group, group of 4 column blocks); column-block groups are padded to a multiple of
   // 8 per group and renumbered so that each XCD (own L2) owns a contiguous run of them for
-  // every token tile of a delta
+  // every token tile of a delta.  xcd_swizzle = 2 ("flat"): units are numbered without the padding, so that workgroup
+  // u, which the hardware places on XCD u % 8, takes column group u % cgs of group u / cgs: a delta's token tiles then
+  // read a column group through different L2s, but every XCD gets the same share of the launch whatever cgs % 8 is
+  // (the host picks it where the padding would leave XCDs short of work).
   const int col_blocks = p.m >> 7;
   const int cgs = (col_blocks + 3) >> 2;
   const int cg_pad = (cgs + 7) & ~7;
   const int unit = blockIdx.x;
   int grp = unit / cg_pad;
-  const int i = unit - grp * cg_pad;
+  int i = unit - grp * cg_pad;
+  const bool flat = p.xcd_swizzle == 2;
+  if (flat) {
+    grp = unit / cgs;
+    i = unit - grp * cgs;
+    if (grp >= p.n_groups * (PLAN_ALL && TOK == 32 && p.tile_halves ? 2 : 1)) return;
+  }
   int half = 0;
   if (PLAN_ALL && TOK == 32 && p.tile_halves) {
     half = grp & 1;
     grp >>= 1;
   }
-  const int cg = p.xcd_swizzle ? (i & 7) * (cg_pad >> 3) + (i >> 3) : i;
+  const int cg = p.xcd_swizzle == 1 ? (i & 7) * (cg_pad >> 3) + (i >> 3) : i;
   if (cg >= cgs) return;
   int delta, start, count;
   bool alt_list = false;

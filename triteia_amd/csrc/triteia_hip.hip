@@ -56,7 +56,7 @@ int check_launch(const char* what) {
 // kUnset marks knobs whose default depends on the launch.
 constexpr int kUnset = -0x7fffffff;
 struct Knobs {
-  int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, pass_nt = 0;
+  int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, flat_min_idle = kUnset, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
   int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1;
@@ -69,7 +69,7 @@ std::once_flag g_knobs_once;
 void read_knobs() {
   Knobs k;
   struct { const char* name; int* dst; } table[] = {
-      {"NT", &k.nt}, {"KW", &k.kw}, {"DEPTH", &k.depth}, {"ROT_SPREAD", &k.rot_spread}, {"XCD_SWIZZLE", &k.xcd_swizzle},
+      {"NT", &k.nt}, {"KW", &k.kw}, {"DEPTH", &k.depth}, {"ROT_SPREAD", &k.rot_spread}, {"XCD_SWIZZLE", &k.xcd_swizzle}, {"FLAT_MIN_IDLE", &k.flat_min_idle},
       {"PASS_NT", &k.pass_nt}, {"WIDE", &k.wide}, {"WIDE_DEPTH", &k.wide_depth}, {"WIDE_MIN_UNITS", &k.wide_min_units},
       {"WIDE_MIN_BATCH", &k.wide_min_batch}, {"PLAN_WIDE_MIN_UNITS", &k.plan_wide_min_units},
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
@@ -270,6 +270,18 @@ constexpr long kWide32KSplitMaxUnits = 256;
 constexpr long kWide64KSplitMaxUnits = 256;
 // Wide (64-token x 512-column) tiles: groups from a plan's wide list or uniform groups.  `tok` = 32: uniform groups
 // in 32-token tiles on the 32-token build with two steps of weights in flight (launches that do not fill the chip).
+// Order of the wide kernel's units over the XCDs.  Column groups padded to a multiple of 8 keep a column group of a
+// delta on one XCD for all its token tiles, but with 28 groups (m = 14336) the eighth XCD gets none of the 32 slots and
+// with 10 (m = 5120) three get none; from three idle slots per tile on, the units are numbered without padding.
+// Measured on plans over deltas of 4096 x 14336 (Zipf(1.2)-routed, padded -> flat): 1024 tokens over 4 / 8 / 16 / 32
+// deltas 118.5 -> 86.0, 118.4 -> 93.2, 128.4 -> 124.7, 202.7 -> 188.8 us, 512 over 32 163.2 -> 149.8 us; evenly routed the
+// same within 2 %.  With 22 groups (m = 11008, two idle slots in 24) flat is the same or slower (cfg3's delta kernel
+// 85.4 -> 89.2 us, at 512 tokens 122.9 -> 129.7 us: its hot delta's tiles then fetch their weights through several L2s).
+constexpr int kFlatUnitsMinIdleSlots = 3;
+static int wide_unit_order(int m) {
+  const int cgs = (m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
+  return knobs().xcd_swizzle == 1 && cg_pad - cgs >= knob_or(knobs().flat_min_idle, kFlatUnitsMinIdleSlots) ? 2 : knobs().xcd_swizzle;
+}
 int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   const long cgs = (a.m / 128 + 3) / 4;
@@ -279,6 +291,7 @@ int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   Sparse24Args b = a;
   if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
+  b.xcd_swizzle = wide_unit_order(a.m);
   if (tok == 32 && units <= knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits))
     hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false, 2>), dim3((unsigned)units), dim3(512), 0, st, b);
   else if (tok == 32)
@@ -902,6 +915,7 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     const int forced = knobs().pass_nt;
     if ((forced == 1 || forced == 2 || forced == 4) && 16 * forced <= tile) pass_nt = forced;
   }
+  if (mid) a.xcd_swizzle = wide_unit_order(prob_m);
   if (mid && mid_big(prob_n, n_deltas, prob_m, prob_k)) {
     // the plan's own list of 64-token tiles, whole, on the 64-token build
     const long cgs = (a.m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
