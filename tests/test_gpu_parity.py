@@ -88,13 +88,18 @@ def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
     out = ops.matmul_4bit_2_4(gq, gx, gm, gs)
     torch.cuda.synchronize()
     check_close(out, ref, what=f"matmul_4bit_2_4 {kernel}")
-    # the units of these small layers are numbered without padding (most of a padded tile's slots would be idle);
-    # with the padded order the same workgroups do the same work on other XCDs
-    setknob(monkeypatch, "TRITEIA_HIP_FLAT_MIN_IDLE", "100")
+    # on these small layers most slots of a padded tile would be idle and the launch puts them to work; the padded order
+    # and the order without padding give the same workgroups the same work on other XCDs
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE_ORDER_MIN_IDLE", "100")
     padded = ops.matmul_4bit_2_4(gq, gx, gm, gs)
     torch.cuda.synchronize()
     assert torch.equal(padded, out), "the order of the units changed bits"
-    delknob(monkeypatch, "TRITEIA_HIP_FLAT_MIN_IDLE")
+    delknob(monkeypatch, "TRITEIA_HIP_WIDE_ORDER_MIN_IDLE")
+    setknob(monkeypatch, "TRITEIA_HIP_XCD_SWIZZLE", "2")
+    unpadded = ops.matmul_4bit_2_4(gq, gx, gm, gs)
+    torch.cuda.synchronize()
+    assert torch.equal(unpadded, out), "the order of the units changed bits"
+    delknob(monkeypatch, "TRITEIA_HIP_XCD_SWIZZLE")
     # same inputs through the narrow kernel: equal up to the order of fp32 accumulation
     setknob(monkeypatch, "TRITEIA_HIP_WIDE", "0")
     narrow = ops.matmul_4bit_2_4(gq, gx, gm, gs)
@@ -689,9 +694,9 @@ def test_plan_lists_64_token_tiles_for_wide_layers(ops, monkeypatch, T, N, k, m,
     assert bool((outs["1"][none] == -3.0).all())
     check_close(torch.where(none[:, None], torch.zeros_like(outs["1"]), outs["1"]), ref, what="64-token tiles beside a 32-token plan")
     assert torch.equal(outs["1"], outs["0"]), "the 64-token tiles changed bits"
-    # (these small layers have their units numbered without padding; the padded order gives the same)
+    # (on these small layers the idle slots of the padding work; the padded order gives the same)
     setknob(monkeypatch, "TRITEIA_HIP_PLAN_BIG", "1")
-    setknob(monkeypatch, "TRITEIA_HIP_FLAT_MIN_IDLE", "100")
+    setknob(monkeypatch, "TRITEIA_HIP_WIDE_ORDER_MIN_IDLE", "100")
     out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
     sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
     torch.cuda.synchronize()

@@ -1,0 +1,66 @@
+"""Orders of the wide kernel's units (sparse24_wide_kernel's first lines, restated): every order gives each
+(tile, column group) to exactly one workgroup of the grid the host launches, and no workgroup looks at a tile past the
+host's bound.  The grid sizes are the library's (triteia_hip_wide_grid_units)."""
+import collections
+
+import pytest
+
+from triteia_amd.python.capi import _ffi
+
+
+def unit_of(u, cgs, rows, order):
+    """(tile, column group) of workgroup u, or None where the kernel returns before it reads a tile."""
+    cg_pad = (cgs + 7) // 8 * 8
+    grp, i = divmod(u, cg_pad)
+    if order == 2:
+        grp, cg = divmod(u, cgs)
+        if grp >= rows:
+            return None
+    elif order == 3:
+        pad = cg_pad - cgs
+        R = (cgs + pad - 1) // pad
+        sg, row = divmod(grp, R)
+        c = (i & 7) * (cg_pad >> 3) + (i >> 3)
+        if c < cgs:
+            grp, cg = sg * (R + 1) + row, c
+        else:
+            grp, cg = sg * (R + 1) + R, row * pad + (c - cgs)
+        if grp >= rows:
+            return None
+    else:
+        cg = (i & 7) * (cg_pad >> 3) + (i >> 3) if order else i
+    if cg >= cgs:
+        return None
+    return grp, cg
+
+
+@pytest.mark.parametrize("order", [0, 1, 2, 3])
+def test_every_unit_once_and_none_past_the_bound(order):
+    lib = _ffi.lib()
+    for cgs in range(1, 41):
+        if order == 3 and cgs % 8 == 0:
+            continue    # no padding: the host never asks for this order
+        m = 512 * cgs
+        for rows in list(range(1, 40)) + [127, 128, 129, 1000]:
+            grid = lib.triteia_hip_wide_grid_units(rows, m, order)
+            seen = collections.Counter()
+            for u in range(grid):
+                t = unit_of(u, cgs, rows, order)
+                if t is not None:
+                    assert 0 <= t[0] < rows, (order, cgs, rows, u, t)
+                    seen[t] += 1
+            assert len(seen) == rows * cgs and set(seen.values()) == {1}, (order, cgs, rows)
+
+
+def test_the_idle_slots_balance_the_xcds():
+    lib = _ffi.lib()
+    for cgs, rows in ((28, 18), (27, 18), (22, 27), (12, 20)):
+        loads = {}
+        for order in (1, 3):
+            load = [0] * 8
+            for u in range(lib.triteia_hip_wide_grid_units(rows, 512 * cgs, order)):
+                if unit_of(u, cgs, rows, order) is not None:
+                    load[u % 8] += 1
+            loads[order] = load
+        assert max(loads[3]) < max(loads[1]), (cgs, rows, loads)
+        assert lib.triteia_hip_wide_unit_order(512 * cgs) == (3 if (cgs + 7) // 8 * 8 - cgs >= 3 else 1)

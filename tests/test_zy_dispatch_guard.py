@@ -61,11 +61,13 @@ ROUTED_GRID = [
 # wide kernel holds two workgroups per CU, the one-deep build three; past the point where the plan's upper bound of tiles
 # fits two per CU, which of them packs the batch's real number of (tile, column group) units into fewer rounds of
 # workgroups depends on the routing (here 858 units: 1.12 rounds of 768 against 1.68 of 512), and only the device has it.
-# The other point: 2048 randomly routed tokens over 16 deltas leave 128 +- 11 per delta, so about half of the deltas spill a
-# few tokens into a third 64-token tile that costs a whole pass over the delta's weights (some 40 tiles x 16 column groups
-# = 640 workgroups, a quarter past the 512 that run together); the split into full 64-token tiles for the wide kernel and
-# rests for the K-split kernel keeps that launch within 512.  Whether a batch spills is again known on the device only.
-KNOWN_GAPS = {(4096, 11008, 32, 512): 1.15, (8192, 8192, 16, 2048): 1.15}
+# The other point: 2048 randomly routed tokens over 16 deltas leave about 120 +- 11 per delta, so some deltas spill a few
+# tokens into a third 64-token tile that costs a whole pass over the delta's weights, and on this layer (16 column groups)
+# 32 tiles are exactly the 512 workgroups that run together: the spill opens a second round.  The split into full
+# 64-token tiles for the wide kernel and rests for the K-split kernel keeps the launch within one round and is 15-19 %
+# ahead here; a host rule for it was measured and is a coin flip (the same split is 15-20 % behind with 8 deltas randomly
+# routed and 4-9 % behind evenly routed, 15 % ahead Zipf-routed): only the device knows whether a batch spills.
+KNOWN_GAPS = {(4096, 11008, 32, 512): 1.15, (8192, 8192, 16, 2048): 1.25}
 # (k, m, tokens): single-matrix products around the windows of the wide kernels and of the K split
 UNIFORM_GRID = [
     (4096, 4096, 16), (4096, 4096, 128), (4096, 4096, 512), (4096, 4096, 640), (4096, 4096, 1024), (4096, 4096, 1536),

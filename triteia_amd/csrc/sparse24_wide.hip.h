@@ -48,29 +48,47 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
 
   // unit = (group, group of 4 column blocks); column-block groups are padded to a multiple of
   // 8 per group and renumbered so that each XCD (own L2) owns a contiguous run of them for
-  // every token tile of a delta.  xcd_swizzle = 2 ("flat"): units are numbered without the padding, so that workgroup
-  // u, which the hardware places on XCD u % 8, takes column group u % cgs of group u / cgs: a delta's token tiles then
-  // read a column group through different L2s, but every XCD gets the same share of the launch whatever cgs % 8 is
-  // (the host picks it where the padding would leave XCDs short of work).
+  // every token tile of a delta.  Where cgs % 8 leaves XCDs short of work, the host asks for one of two other orders
+  // (workgroup u runs on XCD u % 8): xcd_swizzle = 3 puts the idle slots of the padding to work, xcd_swizzle = 2
+  // numbers the units without padding (unit u = column group u % cgs of group u / cgs: balanced, but a delta's token
+  // tiles then read a column group through different L2s).
   const int col_blocks = p.m >> 7;
   const int cgs = (col_blocks + 3) >> 2;
   const int cg_pad = (cgs + 7) & ~7;
   const int unit = blockIdx.x;
   int grp = unit / cg_pad;
   int i = unit - grp * cg_pad;
-  const bool flat = p.xcd_swizzle == 2;
-  if (flat) {
+  const int rows_of_tiles = p.n_groups * (PLAN_ALL && TOK == 32 && p.tile_halves ? 2 : 1);   // the host's bound
+  int cg;
+  if (p.xcd_swizzle == 2) {
     grp = unit / cgs;
-    i = unit - grp * cgs;
-    if (grp >= p.n_groups * (PLAN_ALL && TOK == 32 && p.tile_halves ? 2 : 1)) return;
+    cg = unit - grp * cgs;
+    if (grp >= rows_of_tiles) return;
+  } else if (p.xcd_swizzle == 3) {
+    // padded rows whose idle slots work: R rows of slots serve R + 1 tiles, the last of them through the rows' idle
+    // slots (R * pad >= cgs), so that the XCDs that hold the padding get as many units as the others while all but one
+    // tile in R + 1 keep each column group on one XCD
+    const int pad = cg_pad - cgs;   // > 0: the host asks for this order only then
+    const int R = (cgs + pad - 1) / pad;
+    const int sg = grp / R, row = grp - sg * R;
+    const int c = (i & 7) * (cg_pad >> 3) + (i >> 3);
+    if (c < cgs) {
+      grp = sg * (R + 1) + row;
+      cg = c;
+    } else {
+      grp = sg * (R + 1) + R;
+      cg = row * pad + (c - cgs);
+    }
+    if (grp >= rows_of_tiles) return;
+  } else {
+    cg = p.xcd_swizzle ? (i & 7) * (cg_pad >> 3) + (i >> 3) : i;
   }
+  if (cg >= cgs) return;
   int half = 0;
   if (PLAN_ALL && TOK == 32 && p.tile_halves) {
     half = grp & 1;
     grp >>= 1;
   }
-  const int cg = p.xcd_swizzle == 1 ? (i & 7) * (cg_pad >> 3) + (i >> 3) : i;
-  if (cg >= cgs) return;
   int delta, start, count;
   bool alt_list = false;
   if (p.tiles) {

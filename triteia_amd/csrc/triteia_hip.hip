@@ -56,7 +56,7 @@ int check_launch(const char* what) {
 // kUnset marks knobs whose default depends on the launch.
 constexpr int kUnset = -0x7fffffff;
 struct Knobs {
-  int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, flat_min_idle = kUnset, pass_nt = 0;
+  int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, wide_order_min_idle = kUnset, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
   int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1;
@@ -69,7 +69,7 @@ std::once_flag g_knobs_once;
 void read_knobs() {
   Knobs k;
   struct { const char* name; int* dst; } table[] = {
-      {"NT", &k.nt}, {"KW", &k.kw}, {"DEPTH", &k.depth}, {"ROT_SPREAD", &k.rot_spread}, {"XCD_SWIZZLE", &k.xcd_swizzle}, {"FLAT_MIN_IDLE", &k.flat_min_idle},
+      {"NT", &k.nt}, {"KW", &k.kw}, {"DEPTH", &k.depth}, {"ROT_SPREAD", &k.rot_spread}, {"XCD_SWIZZLE", &k.xcd_swizzle}, {"WIDE_ORDER_MIN_IDLE", &k.wide_order_min_idle},
       {"PASS_NT", &k.pass_nt}, {"WIDE", &k.wide}, {"WIDE_DEPTH", &k.wide_depth}, {"WIDE_MIN_UNITS", &k.wide_min_units},
       {"WIDE_MIN_BATCH", &k.wide_min_batch}, {"PLAN_WIDE_MIN_UNITS", &k.plan_wide_min_units},
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
@@ -270,39 +270,57 @@ constexpr long kWide32KSplitMaxUnits = 256;
 constexpr long kWide64KSplitMaxUnits = 256;
 // Wide (64-token x 512-column) tiles: groups from a plan's wide list or uniform groups.  `tok` = 32: uniform groups
 // in 32-token tiles on the 32-token build with two steps of weights in flight (launches that do not fill the chip).
-// Order of the wide kernel's units over the XCDs.  Column groups padded to a multiple of 8 keep a column group of a
-// delta on one XCD for all its token tiles, but with 28 groups (m = 14336) the eighth XCD gets none of the 32 slots and
-// with 10 (m = 5120) three get none; from three idle slots per tile on, the units are numbered without padding.
-// Measured on plans over deltas of 4096 x 14336 (Zipf(1.2)-routed, padded -> flat): 1024 tokens over 4 / 8 / 16 / 32
-// deltas 118.5 -> 86.0, 118.4 -> 93.2, 128.4 -> 124.7, 202.7 -> 188.8 us, 512 over 32 163.2 -> 149.8 us; evenly routed the
-// same within 2 %.  With 22 groups (m = 11008, two idle slots in 24) flat is the same or slower (cfg3's delta kernel
-// 85.4 -> 89.2 us, at 512 tokens 122.9 -> 129.7 us: its hot delta's tiles then fetch their weights through several L2s).
-constexpr int kFlatUnitsMinIdleSlots = 3;
+// Order of the wide kernel's units over the XCDs (workgroup u runs on XCD u % 8).  Column groups padded to a multiple of
+// 8 keep a column group of a delta on one XCD for all its token tiles, but with 28 groups (m = 14336) the eighth XCD gets
+// none of a tile's 32 slots, with 10 (m = 5120) three get none and with 4 (m = 2048) four.  From three idle slots per
+// tile on, the idle slots are put to work (order 3 of sparse24_wide_kernel: R rows of slots serve R + 1 tiles).
+// Measured, padded -> order 3: plans over deltas of 4096 x 14336, Zipf(1.2)-routed, 1024 tokens over 4 / 8 / 32 deltas
+// 118.5 -> 86.0, 120.7 -> 90.9, 204.8 -> 189.0 us; 5120 x 13824 with 1024 tokens over 8 deltas 145.4 -> 106.8 us; 5120 x 5120
+// with 1024 tokens over 32 deltas 124.6 -> 94.4 us, one matrix with 4096 tokens 178.2 -> 138.6 us; 8192 x 2048, one matrix
+// with 2048 / 4096 tokens 95.9 -> 68.4, 141.1 -> 102.2 us; 4096 x 6144 with 1024 tokens over 8 / 32 deltas 67.3 -> 56.8,
+// 103.3 -> 83.4 us.  Numbering the units without padding (order 2) balances as well but lets every tile of a delta read
+// a column group through another L2: the same on most of these, 4-7 % behind on 5120 x 13824 and 5120 x 5120 (4096 tokens
+// on one matrix 333 against 310 us, 143 against 138 us).  With two idle slots in 24 (m = 11008) neither order gains (cfg3's
+// delta kernel 86.3 -> 87.6-92.7 us with order 3, 85.4 -> 89.2 us with order 2; one matrix with 4096 tokens 218 -> 215 us): its
+// launches fit the three workgroups per CU either way, and the busiest CU decides.
+constexpr int kWideOrderMinIdleSlots = 3;
 static int wide_unit_order(int m) {
   const int cgs = (m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
-  return knobs().xcd_swizzle == 1 && cg_pad - cgs >= knob_or(knobs().flat_min_idle, kFlatUnitsMinIdleSlots) ? 2 : knobs().xcd_swizzle;
+  if (knobs().xcd_swizzle == 3 && cg_pad == cgs) return 1;   // (no padding to put to work)
+  return knobs().xcd_swizzle == 1 && cg_pad - cgs >= knob_or(knobs().wide_order_min_idle, kWideOrderMinIdleSlots) ? 3 : knobs().xcd_swizzle;
+}
+// Workgroups of a wide-kernel launch over `rows` tiles (or halves of tiles) in the given order of units.
+static long wide_grid_units(long rows, int m, int order) {
+  const long cgs = (m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
+  if (order == 2) return rows * cgs;
+  if (order == 3) {
+    const long pad = cg_pad - cgs, R = (cgs + pad - 1) / pad;
+    return (rows / (R + 1) * R + rows % (R + 1)) * cg_pad;
+  }
+  return rows * cg_pad;
 }
 int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   const long cgs = (a.m / 128 + 3) / 4;
   const long cg_pad = (cgs + 7) / 8 * 8;
   const long chunks = a.tiles ? 1 : (a.uniform_count + tok - 1) / tok;
-  const long units = (long)a.n_groups * chunks * cg_pad;
+  const long units = (long)a.n_groups * chunks * cg_pad;   // (the rules below count padded units)
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
   Sparse24Args b = a;
   if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
   b.xcd_swizzle = wide_unit_order(a.m);
+  const unsigned grid = (unsigned)wide_grid_units((long)a.n_groups * chunks, a.m, b.xcd_swizzle);
   if (tok == 32 && units <= knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits))
-    hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false, 2>), dim3((unsigned)units), dim3(512), 0, st, b);
+    hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false, 2>), dim3(grid), dim3(512), 0, st, b);
   else if (tok == 32)
-    hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false>), dim3((unsigned)units), dim3(256), 0, st, b);
+    hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false>), dim3(grid), dim3(256), 0, st, b);
   else if (units <= knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits) &&
            !a.tiles)   // (a plan's launch is sized by an upper bound on its tiles; at 190-230 real units it measured the same either way)
-    hipLaunchKernelGGL((sparse24_wide_kernel<1, kWideTokens, false, 2>), dim3((unsigned)units), dim3(512), 0, st, b);
+    hipLaunchKernelGGL((sparse24_wide_kernel<1, kWideTokens, false, 2>), dim3(grid), dim3(512), 0, st, b);
   else if (knobs().wide_depth == 1)
-    hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3((unsigned)units), dim3(256), 0, st, b);
+    hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3(grid), dim3(256), 0, st, b);
   else
-    hipLaunchKernelGGL((sparse24_wide_kernel<2>), dim3((unsigned)units), dim3(256), 0, st, b);
+    hipLaunchKernelGGL((sparse24_wide_kernel<2>), dim3(grid), dim3(256), 0, st, b);
   return check_launch("sparse24_wide_kernel");
 }
 
@@ -774,6 +792,12 @@ static bool mid_big(int prob_n, int n_deltas, int prob_m, int prob_k) {
   return plan_has_big(prob_n, n_deltas) && (prob_m / 128 + 3) / 4 >= knobs().mid_min_column_groups &&
          mid_tiles(prob_n, n_deltas, prob_m, prob_k) && !mid_deep(prob_n, n_deltas, prob_m, 32);
 }
+int triteia_hip_wide_unit_order(int prob_m) { return prob_m >= 128 ? wide_unit_order(prob_m) : 0; }
+long triteia_hip_wide_grid_units(long rows, int prob_m, int order) {
+  if (rows <= 0 || prob_m < 128) return 0;
+  if (order == 3 && ((prob_m / 128 + 3) / 4) % 8 == 0) order = 1;
+  return wide_grid_units(rows, prob_m, order);
+}
 int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
   if (mid_big(prob_n, n_deltas, prob_m, prob_k)) return 64;
@@ -924,7 +948,7 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     a.n_groups_dev = ws + L.header + 6;
     a.n_groups = L.max_big;
     if ((long)a.n_groups * cg_pad > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units");
-    hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
+    hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3((unsigned)wide_grid_units(a.n_groups, prob_m, a.xcd_swizzle)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), a);
     if (int e = check_launch("sparse24_wide_kernel (plan tiles)")) return e;
   } else if (mid) {
@@ -933,14 +957,14 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     const long units32 = (long)a.n_groups * (tile == 64 ? 2 : 1) * cg_pad;   // in 32-token tiles, on the plan's bound
     if (mid_deep(prob_n, n_deltas, prob_m, tile) && units32 <= 0x7fffffffL) {
       a.tile_halves = tile == 64;
-      hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, true>), dim3((unsigned)units32), dim3(256), 0,
+      hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, true>), dim3((unsigned)wide_grid_units((long)a.n_groups * (tile == 64 ? 2 : 1), prob_m, a.xcd_swizzle)), dim3(256), 0,
                          static_cast<hipStream_t>(stream), a);
       a.tile_halves = 0;
     } else if (tile == 32)
-      hipLaunchKernelGGL((sparse24_wide_kernel<1, 32, true>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
+      hipLaunchKernelGGL((sparse24_wide_kernel<1, 32, true>), dim3((unsigned)wide_grid_units(a.n_groups, prob_m, a.xcd_swizzle)), dim3(256), 0,
                          static_cast<hipStream_t>(stream), a);
     else
-      hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3((unsigned)(a.n_groups * cg_pad)), dim3(256), 0,
+      hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3((unsigned)wide_grid_units(a.n_groups, prob_m, a.xcd_swizzle)), dim3(256), 0,
                          static_cast<hipStream_t>(stream), a);
     if (int e = check_launch("sparse24_wide_kernel (plan tiles)")) return e;
   } else
