@@ -142,6 +142,27 @@ def test_config4_70b_shape(ops, tokens):
     _check_properties(ops, q, me, s, x, wl.indices, range(0, tokens, step), [int(used[0])], f"cfg4 T={tokens}")
 
 
+@pytest.mark.parametrize("k,m,n,tokens,order", [
+    (4096, 14336, 8, 1024, 3),     # Llama-3-8B's MLP: 28 column groups, the padding's idle slots at work
+    (8192, 8192, 16, 2048, 1),     # 16 column groups: the padded order as it is
+    (5120, 13824, 4, 512, 3),      # Llama-2-13B's MLP: 27 column groups
+])
+def test_wide_layers_on_the_plans_64_token_tiles(ops, k, m, n, tokens, order):
+    """Mid-size batches of many tokens per delta on wide layers: the plan is cut in 32-token tiles and also lists
+    64-token tiles, which these layers take on the 64-token build of the wide kernel, in the order of units that
+    suits their number of column groups."""
+    from triteia_amd.python.capi import _ffi
+    lib = _ffi.lib()
+    say(f"64-token list of a 32-token plan k={k} m={m} deltas={n} tokens={tokens}")
+    assert lib.triteia_hip_plan_tile_tokens(tokens, n) == 32
+    assert lib.triteia_hip_planned_tile_kernel(tokens, n, m, k) == 64
+    assert lib.triteia_hip_wide_unit_order(m) == order
+    q, me, s = W.random_packed_deltas(n, k, m, 4100 + n, DEV)
+    x = W.random_activations(tokens, k, 4200 + n, DEV)
+    idx = W.uniform_indices(tokens, n, 4300 + n)
+    _check_properties(ops, q, me, s, x, idx, range(0, tokens, tokens // 5), [0, n - 1], f"{k}x{m} T={tokens}")
+
+
 _CFG4 = {}
 
 
