@@ -178,9 +178,10 @@ TRITEIA_HIP_API size_t triteia_hip_sbmm_routed_static_max_bytes(void);
  *         {tiles, wide} or {all} per weight shape on the device: the wide kernel runs only if
  *         its tiles fill the chip (wide tiles x ceil(prob_m / 512) >= 150, environment
  *         TRITEIA_HIP_PLAN_WIDE_MIN_UNITS); the LoRA path always takes all[].
- *   int32 big[max_big][4]     = for batches of at least 48 tokens per delta (of min(prob_n, n_deltas) deltas) whose
+ *   int32 big[max_big][4]     = for batches of at least 24 tokens per delta (of min(prob_n, n_deltas) deltas) whose
  *         narrow tile size is 32: the same tokens cut into 64-token tiles only (header[6] of them), which wide layers
- *         take on the 64-token build of the wide kernel (environment TRITEIA_HIP_PLAN_BIG=0: never)
+ *         take on the 64-token build of the wide kernel -- from 48 tokens per delta on, or in launches of three rounds
+ *         of workgroups and more (environment TRITEIA_HIP_PLAN_BIG=0: never; above 1: the bar in tokens per delta)
  * with max_tiles = min(prob_n, n_deltas) + prob_n / 16, max_wide = prob_n / 33 + 1 and
  * max_big = min(prob_n, n_deltas) + prob_n / 64.  The
  * narrow tile size is triteia_hip_plan_tile_tokens(prob_n, n_deltas).  Exposed so that one

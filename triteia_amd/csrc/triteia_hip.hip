@@ -783,13 +783,23 @@ static int plan_has_wide(int prob_n, int n_deltas) {
 // 370.9 -> 319.3 us, with 1024 Zipf(1.2)-routed tokens over 8 / 16 deltas 398.6 -> 334.2, 493.7 -> 459.0 us.  With 32 tokens
 // per delta, where every second half of a 64-token tile is empty, it loses (4096 x 11008 with 1024 tokens over 32
 // deltas 122.9 -> 136.8 us), and narrow layers are better off with the workgroups of 32-token tiles.
-constexpr int kPlanBigMinTokensPerDelta = 48;
+// Between 24 and 48 tokens per delta the 64-token tiles pay only where the launch is several rounds of workgroups long
+// (from 2304 units of 32-token tiles on the plan's bound: three rounds), where an empty half here and there no longer
+// decides a round: 8192 x 28672 with 1024 tokens over 24 / 32 deltas, randomly routed 547 -> 502, 634 -> 593 us,
+// Zipf(1.2) 564 -> 546, 693 -> 675 us; on 7B-size layers it is a coin flip at those ratios (4096 x 14336 with 512 tokens
+// over 16 deltas 78 -> 83 us randomly routed, 90 -> 111 us Zipf-routed; 8192 x 8192 with 1024 over 32: 184 -> 165 and
+// 204 -> 222 us).  The plan lists the 64-token tiles from 24 tokens per delta on; each layer decides.
+constexpr int kPlanBigMinTokensPerDelta = 24, kMidBigMinTokensPerDelta = 48;
+constexpr long kMidBigManyUnits = 2304;
 static int plan_has_big(int prob_n, int n_deltas) {
   const long groups = n_deltas < prob_n ? n_deltas : prob_n;
-  return knobs().plan_big && prob_n >= kPlanBigMinTokensPerDelta * groups && triteia_hip_plan_tile_tokens(prob_n, n_deltas) == 32;
+  const long bar = knobs().plan_big == 1 ? kPlanBigMinTokensPerDelta : knobs().plan_big;   // (a knob above 1 is the bar itself)
+  return knobs().plan_big && prob_n >= bar * groups && triteia_hip_plan_tile_tokens(prob_n, n_deltas) == 32;
 }
 static bool mid_big(int prob_n, int n_deltas, int prob_m, int prob_k) {
+  const long groups = n_deltas < prob_n ? n_deltas : prob_n;
   return plan_has_big(prob_n, n_deltas) && (prob_m / 128 + 3) / 4 >= knobs().mid_min_column_groups &&
+         (knobs().plan_big > 1 || prob_n >= kMidBigMinTokensPerDelta * groups || mid_units32(prob_n, n_deltas, prob_m, 32) >= kMidBigManyUnits) &&
          mid_tiles(prob_n, n_deltas, prob_m, prob_k) && !mid_deep(prob_n, n_deltas, prob_m, 32);
 }
 int triteia_hip_wide_unit_order(int prob_m) { return prob_m >= 128 ? wide_unit_order(prob_m) : 0; }
