@@ -48,9 +48,6 @@ def parse():
     p.add_argument("--no-graph", action="store_true", help="time eager launches instead of one captured HIP graph")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-sweep", action="store_true", help="skip the tokens x deltas sweep (the `sweep` array)")
-    p.add_argument("--probe", action="store_true",
-                   help="measure the two ceilings instead: the headline kernel with its MFMAs left out (what memory alone allows for "
-                        "its access pattern) and loops of sparse MFMAs on random operands (what the matrix cores allow)")
     p.add_argument("--warm-cache", action="store_true", help="do not rotate weight copies (Infinity-Cache-warm number)")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also run one plain 256 MiB device copy (a known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -60,20 +57,32 @@ def parse():
 class Problem:
     """Device tensors + bound C-ABI calls for one workload."""
 
-    def __init__(self, wl, copies, torch, ffi):
+    def __init__(self, wl, copies, torch, ffi, weights=None, rotations=1):
+        """`weights`: packed deltas to use instead of drawing `copies` sets of them (several problems on one resident
+        set).  `rotations` (routed sbmm only): step i routes with every index shifted by ((i // copies) % rotations) *
+        (deltas // rotations), modulo the number of deltas -- the same number of distinct deltas and tokens per delta, other
+        deltas: a thin batch on a large resident set then reads cold weights at every step without further copies."""
         from triteia_amd import workloads as W
         self.wl, self.torch, self.ffi = wl, torch, ffi
         dev = "cuda:0"
         self.dev = dev
         self.lib = ffi.lib()
-        self.copies = copies
-        self.weights = [W.random_packed_deltas(wl.n_deltas, wl.k, wl.m, wl.seed + 7919 * c, dev) for c in range(copies)]
+        self.weights = weights if weights is not None else [
+            W.random_packed_deltas(wl.n_deltas, wl.k, wl.m, wl.seed + 7919 * c, dev) for c in range(copies)]
+        self.copies = len(self.weights)
         self.x = W.random_activations(wl.tokens, wl.k, wl.seed + 1, dev)
         self.out = torch.zeros((wl.tokens, wl.m), dtype=torch.float16, device=dev)
         self.idx = torch.from_numpy(wl.indices).to(dev) if wl.indices is not None else None
         nbytes = self.lib.triteia_hip_sbmm_routed_workspace_bytes(wl.tokens, wl.n_deltas)
         self.ws = torch.zeros((nbytes + 3) // 4, dtype=torch.int32, device=dev)
         self.ws_bytes = self.ws.numel() * 4
+        self.rotations = rotations if (wl.op == "sbmm" and wl.indices is not None and not wl.index_offset) else 1
+        self.idx_rot, self.ws_rot = [self.idx], [self.ws]
+        for r in range(1, self.rotations):
+            shift = r * max(1, wl.n_deltas // self.rotations)
+            rot = np.where(wl.indices >= 0, (wl.indices + shift) % wl.n_deltas, wl.indices).astype(np.int32)
+            self.idx_rot.append(torch.from_numpy(rot).to(dev))
+            self.ws_rot.append(torch.zeros_like(self.ws))
         self.lock_ws = torch.zeros(max(wl.m, 16) * max(1, wl.n_deltas), dtype=torch.int32, device=dev)
         # matmul / bmm launches of few workgroups split K across workgroups through a scratch buffer of the caller's
         groups, per_group = (1, wl.tokens) if wl.op == "matmul" else (wl.n_deltas, max(1, wl.tokens // max(1, wl.n_deltas)))
@@ -100,8 +109,9 @@ class Problem:
 
     def plan(self):
         wl, P = self.wl, self.ffi.ptr
-        self._chk(self.lib.triteia_hip_route_plan(P(self.idx), wl.index_offset, wl.n_deltas, wl.tokens, P(self.ws), self.ws_bytes, 0,
-                                                  self.stream()))
+        for idx, ws in zip(self.idx_rot, self.ws_rot):
+            self._chk(self.lib.triteia_hip_route_plan(P(idx), wl.index_offset, wl.n_deltas, wl.tokens, P(ws), self.ws_bytes, 0,
+                                                      self.stream()))
 
     def plan_lora(self):
         """Split index space: the LoRA tokens (indices below index_offset) get a plan of their own."""
@@ -127,7 +137,8 @@ class Problem:
             self._chk(self.lib.triteia_hip_bmm_2_4(P(self.x), P(q), P(me), P(self.out), P(s), wl.m, wl.n_deltas, wl.k, P(self.lock_ws),
                                                     -1, 0, st, -1, -1, -1, 16))
         else:
-            self._chk(self.lib.triteia_hip_sbmm_2_4_planned(P(self.x), P(q), P(me), P(self.out), P(s), P(self.ws), wl.n_deltas, wl.m,
+            ws = self.ws_rot[(i // self.copies) % self.rotations]
+            self._chk(self.lib.triteia_hip_sbmm_2_4_planned(P(self.x), P(q), P(me), P(self.out), P(s), P(ws), wl.n_deltas, wl.m,
                                                             wl.tokens, wl.k, accumulate, 0, st))
 
     def delta_routed(self, i):
@@ -145,8 +156,9 @@ class Problem:
             self.delta_kernel(i)
         elif wl.op == "sbmm":
             q, me, s = self.weights[i % self.copies]
-            self._chk(self.lib.triteia_hip_sbmm_2_4_routed(P(self.x), P(q), P(me), P(self.out), P(s), P(self.idx), 0, wl.n_deltas, wl.m,
-                                                           wl.tokens, wl.k, P(self.ws), self.ws_bytes, 0, 0, self.stream()))
+            r = (i // self.copies) % self.rotations
+            self._chk(self.lib.triteia_hip_sbmm_2_4_routed(P(self.x), P(q), P(me), P(self.out), P(s), P(self.idx_rot[r]), 0, wl.n_deltas,
+                                                           wl.m, wl.tokens, wl.k, P(self.ws_rot[r]), self.ws_bytes, 0, 0, self.stream()))
         elif wl.index_offset:
             # ldmm on a split index space, as triteia_amd.python.ops.ldmm runs it: LoRA plan, zero and shrink beside
             # the base GEMM; then the expand (LoRA rows) beside the routed delta multiply (delta rows)
@@ -300,7 +312,10 @@ def measure(prob, wl, torch, ffi, steps, warmup, use_graph=True, reps=None):
     for i in range(5):
         kernel_call(i)
     torch.cuda.synchronize()
-    batch = 10
+    # one timed batch walks over more distinct weights than the 256 MB Infinity Cache holds (as far as the problem has
+    # them), so that the kernel's duration is a cold one like the step's
+    touched = max(1, wl.distinct_deltas() * wl.delta_bytes)
+    batch = int(max(10, min(prob.copies * prob.rotations, np.ceil(512 * 2 ** 20 / touched))))
     reps = reps or max(3, min(20, steps // 10))
     durs = []
     kgraph = None
@@ -364,6 +379,15 @@ def copies_for(wl, warm=False, asked=0):
     return max(1, min(64, int(np.ceil(1.5 * 2 ** 30 / max(touched, 1))), int(12 * 2 ** 30 // (wl.n_deltas * wl.delta_bytes)) or 1))
 
 
+def rotations_for(wl, copies):
+    """Index rotations (see Problem) that bring a routed sbmm's distinct weights per cycle of steps to about 1.5 GB where
+    the copies alone do not."""
+    if wl.op != "sbmm" or wl.indices is None:
+        return 1
+    touched = max(1, wl.distinct_deltas() * wl.delta_bytes * copies)
+    return int(max(1, min(16, wl.n_deltas // max(1, wl.distinct_deltas()), np.ceil(1.5 * 2 ** 30 / touched))))
+
+
 def sweep_points():
     """The metric's grid: routed sbmm over 16 deltas of 4096 x 4096 and over 32 deltas of 4096 x 11008 against the token
     count, the single-matrix product at three token counts, and the ldmm step of configuration 3."""
@@ -382,10 +406,23 @@ def sweep_points():
     return pts
 
 
+def cfg4_points():
+    """Configuration 4 (Llama-2-70B MLP shape, 64 resident deltas of 8192 x 28672 = 5.64 GB) at its token counts."""
+    from triteia_amd import workloads as W
+    return [(f"sbmm 64 x 8192x28672, {t} tokens Zipf(1.2) (cfg4)", W.config("cfg4", t)) for t in (1, 16, 64, 256, 1024)]
+
+
 def run_sweep(torch, ffi):
+    from triteia_amd import workloads as W
     out = []
-    for label, wl in sweep_points():
-        prob = Problem(wl, copies_for(wl), torch, ffi)
+    points = [(label, wl, None) for label, wl in sweep_points()]
+    # the 5.64 GB of configuration 4 are drawn once and serve its five token counts
+    c4 = cfg4_points()
+    shared = [W.random_packed_deltas(c4[0][1].n_deltas, c4[0][1].k, c4[0][1].m, c4[0][1].seed, "cuda:0")]
+    points += [(label, wl, shared) for label, wl in c4]
+    for label, wl, weights in points:
+        copies = 1 if weights is not None else copies_for(wl)
+        prob = Problem(wl, copies, torch, ffi, weights=weights, rotations=rotations_for(wl, copies))
         torch.cuda.synchronize()
         # a few milliseconds of steps per point
         est_us = max(10.0, wl.delta_flops() / 1.5e15 * 1e6, wl.delta_algorithmic_bytes() / 4e12 * 1e6)
@@ -399,6 +436,8 @@ def run_sweep(torch, ffi):
                     "kernel_us": roof["kernel_us"], "bound": roof["bound"], "frac": roof["frac"]})
         del prob
         torch.cuda.empty_cache()
+    del shared, points
+    torch.cuda.empty_cache()
     return out
 
 
@@ -462,102 +501,6 @@ def measure_lora(torch, ffi, tokens=256, adapters=32, k=4096, m=11008, rank=16, 
     return out
 
 
-def run_probes(torch, ffi):
-    """The ceilings the product kernels are priced against, measured on this GPU (one JSON line)."""
-    from triteia_amd import workloads as W
-    lib, P = ffi.lib(), ffi.ptr
-    wl = W.config("cfg2")
-    prob = Problem(wl, copies_for(wl), torch, ffi)
-    torch.cuda.synchronize()
-
-    def timed(call, batch=10, reps=15):
-        for i in range(5):
-            call(i)
-        torch.cuda.synchronize()
-        durs = []
-        for r in range(reps):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for i in range(batch):
-                call(r * batch + i)
-            e1.record()
-            e1.synchronize()
-            durs.append(e0.elapsed_time(e1) / batch * 1e-3)
-        return float(np.median(durs))
-
-    def loads_only(i):
-        q, me, s = prob.weights[i % prob.copies]
-        prob._chk(lib.triteia_hip_probe_stream(P(prob.x), P(q), P(me), P(prob.out), P(s), P(prob.idx), wl.n_deltas, wl.m, wl.tokens,
-                                               wl.k, 0, prob.stream()))
-
-    t_loads, t_real = timed(loads_only), timed(prob.step)
-    nbytes = wl.delta_algorithmic_bytes()
-    out = {"probe": "ceilings", "workload": wl.name, "algorithmic_bytes": nbytes,
-           "stream": {"kernel": "sparse24_grouped_kernel<1, 4, 1, eager> without its MFMAs", "us": round(t_loads * 1e6, 2),
-                      "gbs": round(nbytes / t_loads / 1e9, 1), "frac_of_8_tbs": round(nbytes / t_loads / 1e9 / HBM_PEAK_GBS, 4)},
-           "product_kernel": {"us": round(t_real * 1e6, 2), "gbs": round(nbytes / t_real / 1e9, 1),
-                              "frac_of_8_tbs": round(nbytes / t_real / 1e9 / HBM_PEAK_GBS, 4), "frac_of_stream_probe": round(t_loads / t_real, 4)}}
-    # what a launch of the same grid costs when it does nothing, and what a plain read of the same packed weights streams at
-    sink1 = torch.zeros(64, dtype=torch.float32, device="cuda:0")
-    grid = 16 * ((wl.m // 128 + 7) // 8 * 8)
-
-    def floor(_i):
-        prob._chk(lib.triteia_hip_probe_launch(grid, P(sink1), 0, prob.stream()))
-
-    def plain_read(i):
-        q = prob.weights[i % prob.copies][0]
-        prob._chk(lib.triteia_hip_probe_read(P(q), q.numel() * q.element_size(), 512, P(sink1), 0, prob.stream()))
-
-    def timed_in_a_graph(call, n=40, reps=7):
-        # launches this short are bound by the host when issued one by one: a captured graph of n of them, replayed
-        for i in range(3):
-            call(i)
-        torch.cuda.synchronize()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            with torch.cuda.graph(graph, stream=side):
-                for i in range(n):
-                    call(i)
-        torch.cuda.synchronize()
-        durs = []
-        for _ in range(reps):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            graph.replay()
-            e1.record()
-            e1.synchronize()
-            durs.append(e0.elapsed_time(e1) / n * 1e-3)
-        del graph
-        return float(np.median(durs))
-
-    t_floor, t_read = timed_in_a_graph(floor), timed_in_a_graph(plain_read)
-    q_bytes = prob.weights[0][0].numel() * prob.weights[0][0].element_size()
-    read_gbs = q_bytes / (t_read - t_floor) / 1e9      # the rate of the streaming itself, the launch's own cost taken off
-    out["launch_floor"] = {"kernel": f"launch_floor_kernel, {grid} workgroups of 256 threads", "us": round(t_floor * 1e6, 2)}
-    out["plain_read"] = {"kernel": "stream_read_kernel, 512 workgroups (the fastest of 512 .. 16384)", "bytes": q_bytes, "us": round(t_read * 1e6, 2),
-                         "gbs_beyond_the_launch": round(read_gbs, 1)}
-    out["product_kernel"]["us_of_a_launch_plus_a_plain_read_of_its_bytes"] = round((t_floor + nbytes / (read_gbs * 1e9)) * 1e6, 2)
-    del prob
-    torch.cuda.empty_cache()
-    src = torch.randn(16384, device="cuda:0").half()
-    sink = torch.empty(256 * 512, dtype=torch.float32, device="cuda:0")
-    iters = 4000
-    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    names = ("32 sparse MFMAs per round, nothing else", "+ 16 LDS reads of 16 bytes per round", "+ 16 LDS reads and 32 conversion pairs per round")
-    out["mfma"] = []
-    for variant, name in enumerate(names):
-        def call(_i, variant=variant):
-            rc = lib.triteia_hip_probe_mfma(variant, iters, P(sink), P(src), 0, stream)
-            assert rc == 0, ffi.last_error()
-        t = timed(call, batch=1, reps=7)
-        flops = 2.0 * 16 * 16 * 64 * 32 * 8 * 256 * iters
-        out["mfma"].append({"loop": name, "ms": round(t * 1e3, 3), "pflops_dense_equivalent": round(flops / t / 1e15, 3),
-                            "frac_of_5_pflops": round(flops / t / 1e15 / 5.0, 4)})
-    print(json.dumps(out))
-
-
 def host_call_us(prob, wl, torch, n=300):
     """Host time of one `ops.sbmm_4bit_2_4_native` call (Python mirror -> ctypes -> C ABI), launches left to queue up."""
     if wl.op != "sbmm":
@@ -588,9 +531,6 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     ffi.lib()   # fails loudly if the HIP library is missing
-    if a.probe:
-        run_probes(torch, ffi)
-        return
 
     shape = tuple(int(v) for v in a.shape.split(",")) if a.shape else None
     if shape is not None and (a.workload != "cfg0" or len(shape) != 2 or shape[0] % 64 or shape[1] % 128):
@@ -601,7 +541,7 @@ def main():
         wl.n_deltas = a.deltas
         wl.indices = W.zipf_indices(wl.tokens, wl.n_deltas, 1.2, wl.seed)
     copies = copies_for(wl, a.warm_cache, a.copies)
-    prob = Problem(wl, copies, torch, ffi)
+    prob = Problem(wl, copies, torch, ffi, rotations=1 if a.warm_cache else rotations_for(wl, copies))
     torch.cuda.synchronize()
     if a.calibrate_copy:
         src = torch.empty(256 * 2 ** 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
@@ -663,6 +603,7 @@ def main():
         "dtype": "f16 (int4 2:4 weights, fp32 accumulate)", "data": "synthetic",
         "config": {"workload": wl.name, "op": wl.op, "k": wl.k, "m": wl.m, "deltas_resident": wl.n_deltas, "deltas_used": wl.distinct_deltas(),
                    "tokens": wl.tokens, "tokens_routed": wl.routed_tokens(), "weight_copies_rotated": copies,
+                   "index_rotations": prob.rotations,
                    "launch": "hip-graph" if use_graph else "eager"},
         "eager_ms_per_step": round(eager / a.steps * 1e3, 5),
         "host_us_per_ops_call": host_call_us(prob, wl, torch),

@@ -213,23 +213,6 @@ TRITEIA_HIP_API long triteia_hip_wide_grid_units(long rows, int prob_m, int orde
  * benchmarks and profiles. */
 TRITEIA_HIP_API int triteia_hip_routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k);
 
-/* Measurement only (bench.py --probe); no counterparts in the reference.
- * triteia_hip_probe_mfma: 256 workgroups x 8 wavefronts issue `iters` rounds of 32 independent
- * v_smfmac_f32_16x16x64_f16 on the random fp16 values at `random_fp16` (>= 16 KB); variant 0: nothing else,
- * 1: + 16 16-byte LDS reads per round, 2: + 16 LDS reads and 32 (bitfield insert, packed add) pairs per round (the
- * operand traffic and int4 -> fp16 conversion of 32 MFMAs when four wavefronts share the dequantised weights).
- * `out`: 512 KiB, overwritten.  2 x 32768 x 32 x 8 x 256 x iters dense-equivalent flops per launch.
- * triteia_hip_probe_stream: the launch that triteia_hip_sbmm_2_4_routed makes for a batch of at most 64 tokens over
- * at most 16 deltas, with the sparse MFMAs left out: same requests, waits, reduction and stores, meaningless values
- * in C.  What the memory system alone allows for that kernel's access pattern. */
-/* triteia_hip_probe_launch: `workgroups` workgroups of 256 threads that start and end (one thread writes out[0]): the cost
- * of a launch.  triteia_hip_probe_read: a plain streaming read of `bytes` bytes at `src` (16-byte aligned, a multiple of
- * 16) by `workgroups` workgroups of 256 threads; `out`: at least 4 bytes of device memory. */
-TRITEIA_HIP_API int triteia_hip_probe_launch(int workgroups, void* out, int dev, void* stream);
-TRITEIA_HIP_API int triteia_hip_probe_read(const void* src, size_t bytes, int workgroups, void* out, int dev, void* stream);
-TRITEIA_HIP_API int triteia_hip_probe_mfma(int variant, int iters, void* out, const void* random_fp16, int dev, void* stream);
-TRITEIA_HIP_API int triteia_hip_probe_stream(const void* A, const void* B, const void* meta, void* C, const void* s, const void* token_indices,
-                             int n_deltas, int prob_m, int prob_n, int prob_k, int dev, void* stream);
 
 /* The multiply step alone, on a plan made by triteia_hip_route_plan for the same
  * (prob_n, n_deltas): C[t] (+)= A[t] @ dequant(B[d]) for every routed token.  One

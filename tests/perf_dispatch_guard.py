@@ -12,7 +12,8 @@ import torch
 from triteia_amd import workloads as W
 from triteia_amd.python.capi import _ffi
 
-pytestmark = pytest.mark.gpu
+# not part of the parity suite (-m gpu): a timing assertion, run by name with -m perf
+pytestmark = pytest.mark.perf
 DEV = "cuda:0"
 TOLERANCE = 1.10
 BIG = "1000000000"

@@ -54,7 +54,7 @@ def test_module_pack_equals_oracle_reference_packer():
     mask = sp.mask_creator(w.t().contiguous())
     w24 = (mask.t() * w).half()
     layer = sparse_low_precision_linear(k, m)
-    layer.pack(w24, s)
+    layer.pack(w24, s, True)
     q = torch.clamp(torch.round(w24 / s).int() + 8, 0, 15)
     if not bool(((q == 0) & mask.t().bool()).any()):
         qo, mo, so = orc.pack_reference(w24.numpy(), s.numpy(), mask=mask.bool().numpy())
@@ -63,7 +63,40 @@ def test_module_pack_equals_oracle_reference_packer():
     W = orc.unpack(layer.qweight.numpy(), layer.meta.numpy(), layer.scale.numpy())
     expect = ((q - 8).half() * s * mask.t()).half()
     assert np.array_equal(W, expect.numpy())
-    layer.pack(w24, s)   # packing twice is allowed
+    layer.pack(w24, s, True)   # packing twice is allowed
+
+
+def test_pack_writes_where_the_reference_writes():
+    """The reference's callers assign `B`, `s` and `meta` on the module and read the packed tensors back from
+    them (generator.py:60-68); `pack` takes `trans` with the reference's default, and that default -- the
+    dense-Marlin permutation, which nothing on this path reads -- raises instead of packing something else."""
+    import inspect
+    from triteia_amd.python.nn.linear import sparse_low_precision_linear
+    g = torch.Generator().manual_seed(19)
+    k, m = 128, 256
+    w = torch.randn((k, m), generator=g).half()
+    s = (w.abs().max(0, keepdim=True)[0] * (2 / 15)).half()
+    mask = sp.mask_creator(w.t().contiguous())
+    w24 = (mask.t() * w).half()
+    assert inspect.signature(sparse_low_precision_linear.pack).parameters["trans"].default is False
+    layer = sparse_low_precision_linear(k, m, groupsize=-1)
+    layer.B = torch.empty((k // 2 // 16, m * 16 // 8), dtype=torch.int)
+    layer.meta = torch.empty((m, k // 16), dtype=torch.int16)
+    layer.s = torch.empty((1, m), dtype=torch.half)
+    with pytest.raises(NotImplementedError, match="trans=True"):
+        layer.pack(w24, s)
+    layer.pack(w24, s, True)
+    plain = sparse_low_precision_linear(k, m)
+    plain.pack(w24, s, True)
+    assert torch.equal(layer.B, plain.qweight) and torch.equal(layer.s, plain.scale) and torch.equal(layer.meta, plain.meta)
+    assert torch.equal(layer.qweight, plain.qweight) and torch.equal(layer.scale, plain.scale)
+    # fp16_to_sparse: the reference's five values; meta_raw is the metadata before the kernel's re-layout
+    out = gen.fp16_to_sparse(w24, s, device="cpu")
+    assert len(out) == 5
+    _, q5, s5, meta5, raw5 = out
+    assert torch.equal(q5, plain.qweight) and torch.equal(meta5, plain.meta) and torch.equal(raw5, plain.meta_raw)
+    assert np.array_equal(orc.reorder_meta(raw5.numpy().view(np.uint16)).view(np.int16), meta5.numpy())
+    assert np.array_equal(orc.unreorder_meta(meta5.numpy().view(np.uint16)).view(np.int16), raw5.numpy())
 
 
 def test_model_distribution():

@@ -19,14 +19,23 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-WIDE_MIN_BATCH = 512          # in these tests plans carry wide tiles from this batch size on ...
+WIDE_MIN_BATCH = 256          # batch size from which a plan carries wide tiles (the library's default)
 
 
-@pytest.fixture(autouse=True)
-def _wide_tiles_from_512_tokens(monkeypatch):
-    setknob(monkeypatch, "TRITEIA_HIP_WIDE_MIN_BATCH", str(WIDE_MIN_BATCH))
-    # ... and the wide kernel takes them however few they are (by default only when they fill the chip)
-    setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
+@pytest.fixture(params=["shipping rules", "wide tiles forced"])
+def plan_rules(request, monkeypatch):
+    """The tests that route through a plan run twice: under the rules as shipped, and with the plan's 64-token wide
+    tiles forced onto these small shapes (carried from 512 tokens on, and taken by the wide kernel however few they
+    are; by default only when they fill the chip)."""
+    global WIDE_MIN_BATCH
+    if request.param == "wide tiles forced":
+        WIDE_MIN_BATCH = 512
+        setknob(monkeypatch, "TRITEIA_HIP_WIDE_MIN_BATCH", str(WIDE_MIN_BATCH))
+        setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
+    else:
+        WIDE_MIN_BATCH = 256
+    yield request.param
+    WIDE_MIN_BATCH = 256
 
 
 def say(msg):
@@ -349,7 +358,7 @@ def _indices(kind, T, N, seed, sort):
     ("zipf", 600, 6, 512, 256, False, 37),           # plan with wide (64-token) tiles
     ("zipf", 700, 5, 640, 192, False, 38),           # the same with a partial last K step
 ])
-def test_sbmm_variants(ops, kind, T, N, m, k, sort, seed):
+def test_sbmm_variants(ops, kind, T, N, m, k, sort, seed, plan_rules):
     say(f"sbmm {kind} T={T} N={N} m={m} k={k} sorted={sort} seed={seed}")
     qw, meta, s = make_deltas(N, k, m, seed)
     x = activations(T, k, seed + 1)
@@ -407,7 +416,7 @@ def _exact_problem(T, N, k, m, seed):
 
 @pytest.mark.parametrize("T,N,k,m,seed", [(64, 16, 512, 384, 51), (37, 5, 1024, 256, 52), (300, 7, 512, 640, 53), (700, 3, 256, 512, 54),
                                           (128, 16, 512, 256, 55), (97, 3, 256, 384, 56), (256, 32, 256, 256, 60), (193, 2, 512, 128, 61)])
-def test_routing_is_bit_exact_on_exact_arithmetic(ops, monkeypatch, T, N, k, m, seed):
+def test_routing_is_bit_exact_on_exact_arithmetic(ops, monkeypatch, T, N, k, m, seed, plan_rules):
     """With inputs on which floating point is exact, every path (fused routing, routing plan with narrow
     and wide tiles, run table, one launch per run, one matmul per delta) must reproduce the oracle bit
     for bit: any token sent to the wrong delta, any row written twice or not at all would show."""
@@ -531,7 +540,7 @@ def test_fused_routing_static_groups(ops, monkeypatch, T, N, used, seed):
     (12000, 3, 256, 128, 92),       # long runs: hundreds of wide tiles per delta, the wide kernel takes them
     (8300, 8192, 128, 128, 93),     # the largest delta count a plan accepts, most deltas without a token
 ])
-def test_large_batches_through_the_plan(ops, T, N, k, m, seed):
+def test_large_batches_through_the_plan(ops, T, N, k, m, seed, plan_rules):
     """Batches beyond the sizes the other tests use: the plan kernel's second pass re-reads the indices
     of tokens past its LDS cache, tile lists are thousands of entries long."""
     say(f"large batch T={T} N={N} k={k} m={m} seed={seed}")
@@ -564,7 +573,7 @@ def test_large_batches_through_the_plan(ops, T, N, k, m, seed):
 
 
 @pytest.mark.parametrize("T,N,k,m,seed", [(64, 1, 512, 384, 95), (150, 2, 256, 640, 96), (100, 1, 320, 128, 97)])
-def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, m, seed):
+def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, m, seed, plan_rules):
     """One or two deltas with tens of tokens on a narrow layer: the plan's 64-token tiles are taken in
     16-token passes split over workgroups.  Same bits as whole tiles (the order of the sums over K does not
     depend on the pass width), within the bar of the oracle."""
@@ -604,7 +613,7 @@ def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, 
     (150, 5, 640, 384, 108, "200"),        # five K steps: the ring of four stages does not end on a whole turn
     (2600, 10, 640, 384, 109, "200"),     # a plan of 64-token tiles, full and ragged (halves with 32, a few and no tokens)
 ])
-def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, seed, wide_bar):
+def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, seed, wide_bar, plan_rules):
     """A plan's 32-token tiles on a wide layer run on the 32-token build of the wide kernel (forced here
     onto small layers).  Against the oracle within the bar; against the K-split kernel within rounding;
     untouched rows stay untouched; accumulation in place."""
@@ -658,7 +667,7 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     (640, 5, 384, 256, 113, (0, 64, 65, 31, 480)),          # no token, a full tile, one over, half a tile, many tiles
     (1024, 16, 128, 128, 114, (64,) * 16),                  # every tile full, one K step, one column block
 ])
-def test_plan_lists_64_token_tiles_for_wide_layers(ops, monkeypatch, T, N, k, m, seed, counts):
+def test_plan_lists_64_token_tiles_for_wide_layers(ops, monkeypatch, T, N, k, m, seed, counts, plan_rules):
     """A batch of 48 tokens per delta and more whose plan is cut in 32-token tiles also lists its tokens in 64-token
     tiles, which wide layers run on the 64-token build of the wide kernel (forced here onto small layers).  Against
     the oracle within the bar; the same bits as from the 32-token tiles; untouched rows stay untouched."""
@@ -703,7 +712,7 @@ def test_plan_lists_64_token_tiles_for_wide_layers(ops, monkeypatch, T, N, k, m,
     assert torch.equal(out, outs["1"]), "the order of the units changed bits"
 
 
-def test_empty_and_degenerate_inputs(ops):
+def test_empty_and_degenerate_inputs(ops, plan_rules):
     """Zero tokens, zero deltas, zero adapters, a batch in which nothing is routed: every op returns the
     shape it should and touches nothing else."""
     say("empty and degenerate inputs")
@@ -735,7 +744,7 @@ def test_empty_and_degenerate_inputs(ops):
     torch.cuda.synchronize()
 
 
-def test_sbmm_with_base_weight_accumulates_in_place(ops):
+def test_sbmm_with_base_weight_accumulates_in_place(ops, plan_rules):
     say("sbmm with base weight")
     T, N, k, m = 24, 4, 256, 256
     qw, meta, s = make_deltas(N, k, m, 41)
@@ -753,7 +762,7 @@ def test_sbmm_with_base_weight_accumulates_in_place(ops):
     assert torch.equal(out[none], torch.matmul(gx, gb.t())[none])
 
 
-def test_route_plan_is_a_stable_grouping():
+def test_route_plan_is_a_stable_grouping(plan_rules):
     from triteia_amd.python.capi import _ffi, route_plan
     say("route plan")
     rng = np.random.default_rng(51)
@@ -881,7 +890,7 @@ def test_lora_ops_bf16(ops, T, M, k, m, r, seed):
     (10, 5, 5, 768, 768, 8, 71), (10, 5, 5, 768, 768, 64, 72),          # tests/ops/test_ldmm.py:103
     (128, 2, 3, 4096, 2048, 16, 73), (128, 16, 16, 1024, 1024, 32, 74),
 ])
-def test_ldmm(ops, T, M, N, m, k, r, seed):
+def test_ldmm(ops, T, M, N, m, k, r, seed, plan_rules):
     say(f"ldmm T={T} M={M} N={N} m={m} k={k} r={r} seed={seed}")
     qw, meta, s = make_deltas(N, k, m, seed)
     A, B = _lora_weights(M, k, r, m, seed + 1, scale=0.05)

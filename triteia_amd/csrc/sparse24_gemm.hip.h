@@ -202,10 +202,7 @@ struct TileCtx {
 // One pass over K for up to 16*NTT tokens of one group: loads, sparse MFMAs, cross-wave
 // reduction, scaled fp16 store.  `first` = index of the pass's first token in the group's list.
 // NPRE: the weights of this wave's first NPRE (<= DEPTH) steps are already on their way in `pre`.
-// PROBE: the same requests, waits and stores with the sparse MFMAs left out (every loaded word is folded into the sums
-// by one integer instruction instead, so that no request can be dropped): what the memory system alone allows for
-// this kernel's access pattern.  Results are meaningless; only the measurement entry point launches it.
-template <int NTT, int KW, int DEPTH, int NPRE = 0, bool PROBE = false>
+template <int NTT, int KW, int DEPTH, int NPRE = 0>
 __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int first, int cnt,
                                           float (*red)[16][kRedStride], int* s_rows, const WPre* pre = nullptr) {
   const int r = c.r, q = c.q, wave = c.wave;
@@ -359,19 +356,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 #pragma unroll
     for (int j = 0; j < DEPTH; j++) {
       const int cur = st + j * KW;
-      if (cur < n_steps) {
-        if (PROBE) {
-          uint32_t fold = 0;
-#pragma unroll
-          for (int a = 0; a < 4; a++) fold ^= ring[j].wq[a][0] ^ ring[j].wq[a][1] ^ ring[j].wq[a][2] ^ ring[j].wq[a][3];
-          fold ^= ring[j].mt[0][0] ^ ring[j].mt[0][3] ^ ring[j].mt[1][0] ^ ring[j].mt[1][3];
-#pragma unroll
-          for (int nt = 0; nt < NTT; nt++) fold ^= ring[j].xa[nt][0][0] ^ ring[j].xa[nt][1][3] ^ ring[j].xb[nt][0][0] ^ ring[j].xb[nt][1][3];
-          acc[0][0][0] += __builtin_bit_cast(float, fold & 0x3f800000u);
-        } else {
-          compute_step(ring[j], cur);
-        }
-      }
+      if (cur < n_steps) compute_step(ring[j], cur);
       load_w(ring[j], cur + DEPTH * KW);
       load_x(ring[j], cur + DEPTH * KW);
     }
@@ -432,7 +417,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 // take the cheaper code path (fewer activation loads and MFMAs) at the same register budget.
 // EAGER: fused routing with group g = delta g (Sparse24Args::raw_static): the weights of the first
 // step are requested at once, together with the indices, instead of one memory round trip later.
-template <int NT, int KW, int DEPTH, bool EAGER = false, bool PROBE = false>
+template <int NT, int KW, int DEPTH, bool EAGER = false>
 __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2 ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
   // steps per wave requested ahead of the routing in the EAGER build (the 32- and 64-token builds
   // also hold narrower passes with a ring of their own depth: one step fits them all)
@@ -612,11 +597,11 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
     // trip to HBM, ahead of the first activation request (measured: 1.8 us between the routing and that request).
     const int cnt = min(count - t0, 16 * NT);
     if (NT == 1 || cnt <= 16) {
-      tile_pass<1, KW, (NT == 1 ? DEPTH : 2), NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
+      tile_pass<1, KW, (NT == 1 ? DEPTH : 2), NPRE>(p, c, start + t0, cnt, red, s_rows, pre);
     } else if (NT == 2 || cnt <= 32) {
-      tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
+      tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), NPRE>(p, c, start + t0, cnt, red, s_rows, pre);
     } else {
-      tile_pass<NT, KW, DEPTH, NPRE, PROBE>(p, c, start + t0, cnt, red, s_rows, pre);
+      tile_pass<NT, KW, DEPTH, NPRE>(p, c, start + t0, cnt, red, s_rows, pre);
     }
     t0 += gridDim.y * 16 * NT;
     if (t0 < count) lds_barrier();    // the next pass over this group's tokens reuses s_rows / red
@@ -624,11 +609,11 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   for (; t0 < count; t0 += gridDim.y * 16 * NT) {
     const int cnt = min(count - t0, 16 * NT);
     if (NT == 1 || cnt <= 16) {
-      tile_pass<1, KW, (NT == 1 ? DEPTH : 2), 0, PROBE>(p, c, start + t0, cnt, red, s_rows);
+      tile_pass<1, KW, (NT == 1 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);
     } else if (NT == 2 || cnt <= 32) {
-      tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), 0, PROBE>(p, c, start + t0, cnt, red, s_rows);
+      tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);
     } else {
-      tile_pass<NT, KW, DEPTH, 0, PROBE>(p, c, start + t0, cnt, red, s_rows);
+      tile_pass<NT, KW, DEPTH>(p, c, start + t0, cnt, red, s_rows);
     }
     // the next pass over this group's tokens reuses s_rows / red
     if (t0 + gridDim.y * 16 * NT < count) lds_barrier();

@@ -11,7 +11,6 @@
 #include <mutex>
 
 #include "lora.hip.h"
-#include "probes.hip.h"
 #include "route_plan.hip.h"
 #include "sparse24_gemm.hip.h"
 #include "sparse24_share.hip.h"
@@ -287,7 +286,8 @@ constexpr int kWideOrderMinIdleSlots = 3;
 static int wide_unit_order(int m) {
   const int cgs = (m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
   if (knobs().xcd_swizzle == 3 && cg_pad == cgs) return 1;   // (no padding to put to work)
-  return knobs().xcd_swizzle == 1 && cg_pad - cgs >= knob_or(knobs().wide_order_min_idle, kWideOrderMinIdleSlots) ? 3 : knobs().xcd_swizzle;
+  // (order 3 divides by the number of padding slots: never without any, whatever the knob says)
+  return knobs().xcd_swizzle == 1 && cg_pad > cgs && cg_pad - cgs >= knob_or(knobs().wide_order_min_idle, kWideOrderMinIdleSlots) ? 3 : knobs().xcd_swizzle;
 }
 // Workgroups of a wide-kernel launch over `rows` tiles (or halves of tiles) in the given order of units.
 static long wide_grid_units(long rows, int m, int order) {
@@ -814,61 +814,6 @@ int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int pr
   return mid_tiles(prob_n, n_deltas, prob_m, prob_k) ? triteia_hip_plan_tile_tokens(prob_n, n_deltas) : 0;
 }
 
-int triteia_hip_probe_mfma(int variant, int iters, void* out, const void* random_fp16, int dev, void* stream) {
-  if (iters <= 0 || !out || !random_fp16) return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_mfma: iters=%d or a null buffer", iters);
-  DeviceGuard g(dev);
-  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  float* o = static_cast<float*>(out);
-  const _Float16* src = static_cast<const _Float16*>(random_fp16);
-  if (variant == 0) hipLaunchKernelGGL((mfma_probe_kernel<0, 0>), dim3(256), dim3(512), 0, st, iters, o, src);
-  else if (variant == 1) hipLaunchKernelGGL((mfma_probe_kernel<16, 0>), dim3(256), dim3(512), 0, st, iters, o, src);
-  else if (variant == 2) hipLaunchKernelGGL((mfma_probe_kernel<16, 32>), dim3(256), dim3(512), 0, st, iters, o, src);
-  else return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_mfma: variant %d", variant);
-  return check_launch("mfma_probe_kernel");
-}
-
-int triteia_hip_probe_launch(int workgroups, void* out, int dev, void* stream) {
-  if (workgroups <= 0 || workgroups > (1 << 20) || !out) return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_launch: workgroups=%d or a null buffer", workgroups);
-  DeviceGuard g(dev);
-  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
-  hipLaunchKernelGGL(launch_floor_kernel, dim3((unsigned)workgroups), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<float*>(out));
-  return check_launch("launch_floor_kernel");
-}
-
-int triteia_hip_probe_read(const void* src, size_t bytes, int workgroups, void* out, int dev, void* stream) {
-  if (workgroups <= 0 || workgroups > (1 << 20) || !out || !src || bytes % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0)
-    return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_read: needs a 16-byte aligned buffer of a multiple of 16 bytes and 1 .. 2^20 workgroups");
-  DeviceGuard g(dev);
-  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
-  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint4_t*>(src), (long)(bytes / 16), static_cast<float*>(out));
-  return check_launch("stream_read_kernel");
-}
-
-int triteia_hip_probe_stream(const void* A, const void* B, const void* meta, void* C, const void* s, const void* token_indices,
-                             int n_deltas, int prob_m, int prob_n, int prob_k, int dev, void* stream) {
-  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, -1)) return e;
-  if (prob_n <= 0 || prob_n > 64 || n_deltas <= 0 || n_deltas > 16 || !A || !B || !meta || !C || !s || !token_indices)
-    return fail(TRITEIA_HIP_ERR_ARGUMENT, "probe_stream: at most 64 tokens over at most 16 deltas, no null pointers");
-  DeviceGuard g(dev);
-  if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
-  // the launch of triteia_hip_sbmm_2_4_routed for such a batch (in-kernel routing, weights requested ahead of it)
-  Sparse24Args a;
-  fill_weights(a, A, B, meta, C, s, prob_m, prob_k, n_deltas);
-  a.raw_indices = static_cast<const int*>(token_indices);
-  a.raw_count = prob_n;
-  a.n_groups = n_deltas;
-  a.raw_static = 1;
-  const long cb_pad = (a.m / 128 + 7) / 8 * 8;
-  const long side_by_side = 512 / cb_pad;
-  const int n_steps = (a.k / 32 + 3) / 4;
-  a.rot_spread = side_by_side >= 4 ? (int)(n_steps / (side_by_side < 16 ? side_by_side : 16)) : 0;
-  hipLaunchKernelGGL((sparse24_grouped_kernel<1, 4, 1, true, true>), dim3((unsigned)(n_deltas * cb_pad)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), a);
-  return check_launch("sparse24_grouped_kernel (loads only)");
-}
-
 int triteia_hip_routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
   if (!routed_in_kernel(prob_n, n_deltas, prob_m, prob_k)) return 0;
@@ -995,6 +940,7 @@ int triteia_hip_sbmm_2_4_routed(const void* A, const void* B, const void* meta, 
                                 void* stream) {
   if (int e = check_gemm_shape(prob_m, prob_n, prob_k, -1)) return e;
   if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: accumulate=%d", accumulate);
+  if (n_deltas < 0) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sbmm_2_4_routed: deltas=%d", n_deltas);
   if (prob_m == 0 || prob_n == 0 || prob_k == 0 || n_deltas == 0) return TRITEIA_HIP_OK;
   if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sbmm_2_4_routed: null tensor pointer");
   // (above 64 tokens only for at most 16 deltas, whose weights can be requested ahead of the routing: with 32 deltas of

@@ -37,10 +37,6 @@ SIGNATURES = {
     "triteia_hip_sbmm_2_4_planned": (_c_int, [_c_vp] * 6 + [_c_int] * 5 + [_c_int, _c_vp]),
     "triteia_hip_sbmm_routed_workspace_bytes": (_c_sz, [_c_int, _c_int]),
     "triteia_hip_plan_tile_tokens": (_c_int, [_c_int, _c_int]),
-    "triteia_hip_probe_launch": (_c_int, [_c_int, _c_vp, _c_int, _c_vp]),
-    "triteia_hip_probe_read": (_c_int, [_c_vp, ctypes.c_size_t, _c_int, _c_vp, _c_int, _c_vp]),
-    "triteia_hip_probe_mfma": (_c_int, [_c_int, _c_int, _c_vp, _c_vp, _c_int, _c_vp]),
-    "triteia_hip_probe_stream": (_c_int, [_c_vp] * 6 + [_c_int] * 4 + [_c_int, _c_vp]),
     "triteia_hip_routed_in_kernel": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
     "triteia_hip_planned_tile_kernel": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
     "triteia_hip_wide_unit_order": (_c_int, [_c_int]),
@@ -120,18 +116,27 @@ def require_dtype(t, dtype, name):
         raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
 
 
-_SPLIT_SCRATCH = {}
+_SPLIT_SCRATCH = {}          # (device, stream) -> buffer, most recently created last
+_SPLIT_SCRATCH_MAX_STREAMS = 16
 
 
 def split_scratch(nbytes: int, device) -> torch.Tensor:
     """Scratch for the K split of small matmul / bmm launches (fp32 partial sums): one buffer per device and
-    stream, grown on demand, so that calls on different streams never share one."""
+    stream, grown on demand, so that calls on different streams never share one; the streams seen longest ago
+    give theirs up once more than a handful have asked.  A call recorded into a graph gets a buffer of its own
+    from the graph's memory pool, which is not kept: it belongs to that graph, not to later calls on the stream."""
     dev = torch.device(device)
+    nbytes = (int(nbytes) + 255) // 256 * 256
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
     buf = _SPLIT_SCRATCH.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(int(nbytes), 4 << 20), dtype=torch.uint8, device=dev)
+        buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        _SPLIT_SCRATCH.pop(key, None)
         _SPLIT_SCRATCH[key] = buf
+        while len(_SPLIT_SCRATCH) > _SPLIT_SCRATCH_MAX_STREAMS:
+            _SPLIT_SCRATCH.pop(next(iter(_SPLIT_SCRATCH)))
     return buf
 
 

@@ -2,7 +2,7 @@ import torch
 import torch.nn as nn
 
 from triteia_amd.python.capi import mul_2_4
-from triteia_amd.python.ops.utils.sparsity import mask_creator, pack_2_4, positions_from_mask
+from triteia_amd.python.ops.utils.sparsity import mask_creator, meta_raw, pack_2_4, positions_from_mask
 
 
 class sparse_low_precision_linear(nn.Module):
@@ -32,18 +32,28 @@ class sparse_low_precision_linear(nn.Module):
         return C
 
     @torch.no_grad()
-    def pack(self, weight, scales, trans=True):
-        """Quantise and pack `weight` [k, m] fp16 with per-column `scales` [1, m] into the
-        module's buffers.  The kept 2-of-4 positions come from the magnitude mask, not from
-        `!= 0`, so a kept value that quantises to -8 stays where it was.  Unlike the reference
-        (linear.py:125-126) the module's attributes are left intact and can be packed again."""
+    def pack(self, weight, scales, trans=False):
+        """Quantise and pack `weight` [k, m] fp16 with per-column `scales` [1, m] (linear.py:79-141).
+
+        Signature and destinations are the reference's: `trans=True` selects the 2:4 layout the kernels read
+        (every call site of the reference passes it: generator.py:66,120,173); the default, `trans=False`, is
+        the dense-Marlin permutation, which no kernel of this path consumes, and raises.  The result goes where
+        the reference puts it -- the attributes `B`, `s` and `meta` that its callers assign beforehand
+        (generator.py:60-65), when they exist -- and also into the registered buffers `qweight`, `scale`,
+        `meta`, so that `forward` works on a module packed either way; `meta_raw` holds the metadata before
+        the kernel's re-layout.  The kept 2-of-4 positions come from the magnitude mask, not from `!= 0`,
+        so a kept value that quantises to -8 stays where it was.  Unlike the reference (linear.py:125-126)
+        `infeatures` and `groupsize` are left intact and the module can be packed again."""
         if weight.dtype != torch.half:
             raise ValueError("Only `torch.half` weights are supported.")
         if not trans:
-            raise NotImplementedError("only the 2:4 layout (trans=True) is implemented")
+            raise NotImplementedError(
+                "pack(..., trans=False) asks for the dense-Marlin permutation of the compressed weight, a layout that "
+                "no kernel of this path reads; pass trans=True for the 2:4 layout (as every caller in the reference does)")
         k, m = weight.shape
         assert (k, m) == (self.infeatures, self.outfeatures)
-        dev = self.qweight.device
+        B, s_attr = getattr(self, "B", None), getattr(self, "s", None)
+        dev = B.device if isinstance(B, torch.Tensor) else self.qweight.device
         w = weight.to(dev)
         s = scales.to(dev).reshape(1, m)
         mask = mask_creator(w.t().contiguous(), n=2, m=4)
@@ -53,8 +63,13 @@ class sparse_low_precision_linear(nn.Module):
         kept = torch.stack([qt.gather(-1, lo.unsqueeze(-1)).squeeze(-1), qt.gather(-1, hi.unsqueeze(-1)).squeeze(-1)], -1)
         qweight, meta, s16 = pack_2_4(kept.reshape(m, k // 2), lo, hi, s)
         self.qweight.copy_(qweight)
-        self.meta.copy_(meta)
+        self.meta.copy_(meta)        # (the buffer, or the tensor a caller has put in its place)
         self.scale.copy_(s16)
+        if isinstance(B, torch.Tensor):
+            B[:, :] = qweight.to(B.device)
+        if isinstance(s_attr, torch.Tensor):
+            s_attr[:, :] = s16.to(s_attr.device)
+        self.meta_raw = meta_raw(lo, hi)
 
 
 class multi_delta_linear(nn.Module):
@@ -91,7 +106,7 @@ class multi_delta_linear(nn.Module):
     def pack_delta(self, i, weight, scales):
         """Quantise and pack a dense [k, m] fp16 delta with per-column scales into slot i."""
         layer = sparse_low_precision_linear(self.infeatures, self.outfeatures).to(self.qweight.device)
-        layer.pack(weight, scales)
+        layer.pack(weight, scales, True)
         self.load_delta(i, layer)
 
     def forward(self, x, indices, plan=None):

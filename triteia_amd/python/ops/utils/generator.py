@@ -9,7 +9,7 @@ and packing records the kept positions explicitly, so a kept value of -8
 import numpy as np
 import torch
 
-from .sparsity import mask_creator, pack_2_4, positions_from_mask
+from .sparsity import mask_creator, meta_raw, pack_2_4, positions_from_mask
 
 
 def _randn(shape, generator, device, dtype=torch.float16):
@@ -30,8 +30,8 @@ def gen_batched_lora_16_bit(b, m, n, rank, device="cuda", generator=None):
 def fp16_to_sparse(weights, scale, device="cuda", mask=None):
     """Quantise + pack a [k, m] fp16 weight that is (to be made) 2:4 sparse along k.
 
-    Returns (weights, qweight, scales, meta) like the reference's fp16_to_sparse minus its
-    `meta_raw` debugging output."""
+    Returns (weights, qweight, scales, meta, meta_raw), the reference's five values (generator.py:105-123);
+    `meta_raw` is the metadata before the kernel's re-layout: int16 [m, k/16], row = output column."""
     weights = weights.to(device)
     scale = scale.to(device).reshape(1, -1)
     k, m = weights.shape
@@ -42,7 +42,7 @@ def fp16_to_sparse(weights, scale, device="cuda", mask=None):
     qt = q.t().reshape(m, k // 4, 4)
     kept = torch.stack([qt.gather(-1, lo.unsqueeze(-1)).squeeze(-1), qt.gather(-1, hi.unsqueeze(-1)).squeeze(-1)], -1)
     qweight, meta, s = pack_2_4(kept.reshape(m, k // 2), lo, hi, scale)
-    return weights, qweight, s, meta
+    return weights, qweight, s, meta, meta_raw(lo, hi)
 
 
 def gen_sparse_quant4_NT(m, k, groupsize=-1, device="cuda", prune_n=2, prune_m=4, generator=None):
@@ -62,7 +62,7 @@ def gen_sparse_quant4_NT(m, k, groupsize=-1, device="cuda", prune_n=2, prune_m=4
     ref = (wq - (maxq + 1) // 2).half() * s
     mask = mask_creator(wq.t().contiguous(), n=prune_n, m=prune_m)  # on the shifted codes, as the reference does
     uncompress = (mask.to(ref.dtype) * ref.t()).t().contiguous()
-    _, q, s_out, meta = fp16_to_sparse(uncompress, s, device=device, mask=mask)
+    _, q, s_out, meta, _ = fp16_to_sparse(uncompress, s, device=device, mask=mask)
     return uncompress, q, s_out, meta
 
 
@@ -133,7 +133,7 @@ def torch_weight_to_sparse_marlin(weight, scale, tp_size=1, chunk_by="column", d
         else:
             lo_r, hi_r = i * weight.size(0) // tp_size, (i + 1) * weight.size(0) // tp_size
             tp_weight, tp_scales = weight[lo_r:hi_r, :], scale
-        _, q, s, meta = fp16_to_sparse(tp_weight.contiguous(), tp_scales.contiguous(), device=device)
+        _, q, s, meta, _ = fp16_to_sparse(tp_weight.contiguous(), tp_scales.contiguous(), device=device)
         qweights.append(q.contiguous())
         scales.append(s.contiguous())
         metas.append(meta.contiguous())

@@ -79,13 +79,27 @@ def unpack_nibbles(qweight: torch.Tensor) -> torch.Tensor:
     return t.reshape(kt * 16, m).to(torch.uint8)
 
 
+def _meta_words(lo: torch.Tensor, hi: torch.Tensor) -> torch.Tensor:
+    """Kept positions (lo < hi) [m, k/4] -> the 16-bit metadata words as int64 [m, k/16], word (r, c) = the four
+    (lo | hi << 2) codes of column r in 16-k block c, low bits first (logical order, before any re-layout)."""
+    m, kg = lo.shape
+    code = (lo.to(torch.int64) | (hi.to(torch.int64) << 2)).reshape(m, kg // 4, 4)
+    return code[..., 0] | (code[..., 1] << 4) | (code[..., 2] << 8) | (code[..., 3] << 12)
+
+
+def meta_raw(lo: torch.Tensor, hi: torch.Tensor) -> torch.Tensor:
+    """The metadata words int16 [m, k/16] in logical order: row = output column, column = 16-k block (what the
+    CUTLASS-style compressor yields before the kernel's re-layout, triteia/python/ops/utils/sparsity.py:220-244)."""
+    w16 = _meta_words(lo, hi)
+    return torch.where(w16 >= 2 ** 15, w16 - 2 ** 16, w16).to(torch.int16)
+
+
 def pack_meta(lo: torch.Tensor, hi: torch.Tensor) -> torch.Tensor:
     """Kept positions (lo < hi) [m, k/4] -> metadata int16 [m, k/16] in physical order."""
     m, kg = lo.shape
     if m % 64 != 0 or kg % 8 != 0:
         raise ValueError("need m % 64 == 0 and k % 32 == 0")
-    code = (lo.to(torch.int64) | (hi.to(torch.int64) << 2)).reshape(m, kg // 4, 4)
-    w16 = code[..., 0] | (code[..., 1] << 4) | (code[..., 2] << 8) | (code[..., 3] << 12)   # [m, k/16]
+    w16 = _meta_words(lo, hi)                                   # [m, k/16]
     t = w16.reshape(m // 64, 2, 2, 2, 2, 2, 2, kg // 8, 2)     # R b5 b4 b3 b2 b1 b0 tr h
     t = t.permute(7, 0, 5, 1, 2, 3, 6, 8, 4)                    # tr R b1 b5 b4 b3 b0 h b2
     t = t.reshape(m, kg // 4)
