@@ -235,6 +235,13 @@ TRITEIA_HIP_API int triteia_hip_bgmv(void* Y, const void* X, const void* W, cons
  * (triteia/csrc/ops/bgmv_all.cu:4-5) and dispatches on the tensors' dtype (ops.cpp:199-214). */
 TRITEIA_HIP_API int triteia_hip_bgmv_bf16(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
                           int num_layers, int layer_idx, float scale, int dev, void* stream);
+/* Y[b, :] = scale * W[...] @ X[b, :]: the same product stored instead of added (Y is not read; rows with a negative
+ * index are left as they are).  No counterpart in the reference, whose add_lora_bgmv clears a [batch, rank]
+ * intermediate and adds into it (triteia/python/capi/punica.py:59-68): with this form the intermediate needs no clearing. */
+TRITEIA_HIP_API int triteia_hip_bgmv_store(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                           int num_layers, int layer_idx, float scale, int dev, void* stream);
+TRITEIA_HIP_API int triteia_hip_bgmv_store_bf16(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                                int num_layers, int layer_idx, float scale, int dev, void* stream);
 
 /* SGMV: y[s[i] : s[i+1]] += x[s[i] : s[i+1]] @ W_i, W_i = (fp16*)w_ptrs[i] +
  * layer_idx * d_in * d_out, row-major [d_in, d_out]; s int32 [num_problems+1].
@@ -248,21 +255,29 @@ TRITEIA_HIP_API size_t triteia_hip_sgmv_tmp_size(int num_problems); /* reference
  * dispatched on x's dtype, ops.cpp:132-143). */
 TRITEIA_HIP_API int triteia_hip_sgmv_bf16(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
                           int d_out, int layer_idx, int dev, void* stream);
+/* y[s[i] : s[i+1]] = x[s[i] : s[i+1]] @ W_i: the same product stored instead of added (y is not read; rows outside
+ * every segment are left as they are).  No counterpart in the reference, whose add_lora_sgmv_cutlass clears the
+ * [rows, rank] intermediate first (triteia/python/capi/punica.py:30-57). */
+TRITEIA_HIP_API int triteia_hip_sgmv_store(void* y, const void* x, const void* w_ptrs, const void* s, int num_problems, int d_in, int d_out,
+                           int layer_idx, int dev, void* stream);
+TRITEIA_HIP_API int triteia_hip_sgmv_store_bf16(void* y, const void* x, const void* w_ptrs, const void* s, int num_problems, int d_in, int d_out,
+                                int layer_idx, int dev, void* stream);
 
 /* Routed SGMV on a routing plan made by triteia_hip_route_plan: for every group
  * g (adapter a = g_delta[g]) and every listed row t:
- *   y[t] += scale * x[t] @ W[a],  W = w_base + a * w_stride (elements),
- *   row-major [d_in, d_out].
+ *   y[t] (+)= scale * x[t] @ W[a],  W = w_base + a * w_stride (elements),
+ *   row-major [d_in, d_out]; accumulate = 1 adds to y, 0 stores (y is not read, rows
+ *   that the plan does not list are left as they are).
  * No counterpart in the reference, which builds the segment table on the host
  * (triteia/python/ops/matmul/lora.py:63-96). */
 TRITEIA_HIP_API int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
                             int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
-                            int dev, void* stream);
+                            int accumulate, int dev, void* stream);
 
 /* The same for bf16 tensors (y, x, w_base). */
 TRITEIA_HIP_API int triteia_hip_sgmv_routed_bf16(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
                                  int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
-                                 int dev, void* stream);
+                                 int accumulate, int dev, void* stream);
 
 #ifdef __cplusplus
 }

@@ -859,6 +859,55 @@ def test_lora_ops(ops, T, M, k, m, r, seed):
     check_close(ops.lora_sgmv_routed(gA, gB, gx2, gi2), ref2, what="lora_sgmv_routed unsorted")
 
 
+@pytest.mark.parametrize("T,M,d_in,d_out,seed", [
+    (37, 4, 1024, 16, 171), (37, 4, 16, 1024, 172), (90, 3, 512, 64, 173), (90, 3, 64, 520, 174), (20, 2, 768, 128, 175),
+    (64, 5, 32, 2048, 176), (50, 3, 24, 256, 177),
+])
+def test_lora_kernels_store_instead_of_add(T, M, d_in, d_out, seed):
+    """The stored form of BGMV / SGMV / routed SGMV (no counterpart in the reference; the intermediate of a LoRA pair then
+    needs no clearing): rows that take an adapter hold the product alone, whatever the output held before; the others
+    keep what they held.  Both directions (wide -> narrow, narrow -> wide), against a plain fp32 product."""
+    from triteia_amd.python.capi import route_plan, sgmv_routed
+    from triteia_amd.python.capi.punica import dispatch_bgmv, sgmv, sgmv_tmp_size
+    say(f"lora store T={T} M={M} d_in={d_in} d_out={d_out} seed={seed}")
+    rng = np.random.default_rng(seed)
+    W = (rng.standard_normal((M, d_in, d_out)) * 0.1).astype(np.float16)
+    x = (rng.standard_normal((T, d_in))).astype(np.float16)
+    idx = np.sort(rng.integers(-1, M, size=T)).astype(np.int32)
+    ref = np.full((T, d_out), 7.0)
+    for t in range(T):
+        if idx[t] >= 0:
+            ref[t] = x[t].astype(np.float64) @ W[idx[t]].astype(np.float64)
+    gW, gx, gi = to_gpu(W, x, idx)
+    routed = torch.from_numpy(idx >= 0).to(DEV)
+
+    def check(y, what):
+        torch.cuda.synchronize()
+        assert bool((y[~routed] == 7).all()), what + ": a row without an adapter was written"
+        check_close(y[routed], ref[idx >= 0], tol=2e-3, what=what)
+
+    y = torch.full((T, d_out), 7.0, dtype=torch.float16, device=DEV)
+    sgmv_routed(y, gx, gW, route_plan(gi, M), accumulate=False)
+    check(y, "routed SGMV, stored")
+    y = torch.full((T, d_out), 7.0, dtype=torch.float16, device=DEV)
+    dispatch_bgmv(y, gx, gW.transpose(1, 2).contiguous().unsqueeze(1), gi.to(torch.long), 0, 1.0, accumulate=False)
+    check(y, "BGMV, stored")
+    # SGMV on a segment table: rows of the leading -1 run lie outside every segment
+    y = torch.full((T, d_out), 7.0, dtype=torch.float16, device=DEV)
+    skip = int((idx < 0).sum())
+    counts = np.bincount(idx[idx >= 0], minlength=M)
+    seg = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)).to(DEV)
+    w_ptr = torch.tensor([gW[i].data_ptr() for i in range(M)], dtype=torch.int64, device=DEV)
+    tmp = torch.empty((sgmv_tmp_size(M),), dtype=torch.uint8, device=DEV)
+    sgmv(y[skip:], gx[skip:], w_ptr, seg, tmp, 0, accumulate=False)
+    check(y, "SGMV, stored")
+    # and added on top of what is there, as before
+    y = torch.full((T, d_out), 7.0, dtype=torch.float16, device=DEV)
+    sgmv_routed(y, gx, gW, route_plan(gi, M))
+    torch.cuda.synchronize()
+    check_close(y[routed].float() - 7.0, ref[idx >= 0], tol=2e-2, what="routed SGMV, added")
+
+
 @pytest.mark.parametrize("T,M,k,m,r,seed", [
     (10, 5, 768, 256, 64, 161), (33, 4, 512, 1024, 16, 162), (71, 3, 512, 520, 24, 163), (41, 2, 1024, 512, 128, 164),
 ])

@@ -46,7 +46,9 @@ __device__ __forceinline__ float wave_sum(float v) {
 // 8-element pieces t, t + 256, ... of x and of each of the 16 weight rows (all of a piece's loads are independent, so
 // they are in flight together), then the 16 partial sums are added over the wavefront by shuffles and over the four
 // wavefronts through LDS.
-template <class T>
+// ACC: the result is added to what Y holds (the reference's semantics); otherwise it is stored, and Y is not read
+// (rows whose index is negative are left alone either way).
+template <class T, bool ACC = true>
 __global__ __launch_bounds__(256) void bgmv_shrink_kernel(T* __restrict__ Y, const T* __restrict__ X,
                                                          const T* __restrict__ W,
                                                          const long long* __restrict__ indices, int h_in, int h_out,
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(T* __restrict__ Y, con
     if (threadIdx.x < n_out) {
       const float sum = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
       T* yp = Y + (long)b * h_out + oc + threadIdx.x;
-      *yp = (T)((float)*yp + sum * scale);
+      *yp = (T)((ACC ? (float)*yp : 0.f) + sum * scale);
     }
     __syncthreads();
   }
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(T* __restrict__ Y, con
 // narrow -> wide: grid (ceil(h_out / 2048), B), block 256.  A thread owns 8 consecutive outputs: their 8 weight rows are
 // one contiguous piece of memory (h_in elements each), the token's h_in activations are the same address in every lane,
 // and the old outputs are one 16-byte load; everything is requested before the first result is used.
-template <class T>
+template <class T, bool ACC = true>
 __global__ __launch_bounds__(256) void bgmv_expand_kernel(T* __restrict__ Y, const T* __restrict__ X,
                                                          const T* __restrict__ W,
                                                          const long long* __restrict__ indices, int h_in, int h_out,
@@ -105,7 +107,8 @@ __global__ __launch_bounds__(256) void bgmv_expand_kernel(T* __restrict__ Y, con
   const T* w = W + ((idx * num_layers + layer_idx) * (long)h_out + j0) * h_in;
   const T* x = X + (long)b * h_in;
   T* yp = Y + (long)b * h_out + j0;
-  const lvec8<T> old = *reinterpret_cast<const lvec8<T>*>(yp);
+  lvec8<T> old = lvec8<T>{0, 0, 0, 0, 0, 0, 0, 0};
+  if (ACC) old = *reinterpret_cast<const lvec8<T>*>(yp);
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; e++) acc[e] = 0.f;
@@ -133,7 +136,7 @@ __global__ __launch_bounds__(256) void bgmv_expand_kernel(T* __restrict__ Y, con
 // updates the output.  A block takes TB consecutive tokens; the weights stay in registers from one token to the next
 // and are fetched again only when the adapter changes (sorted batches, the hot adapter of a skewed one).
 // grid (ceil(h_out / (4 Q 64 / LPR)), ceil(B / TB)), block 256.
-template <class T, int LPR, int Q, int TB>
+template <class T, int LPR, int Q, int TB, bool ACC = true>
 __global__ __launch_bounds__(256) void bgmv_expand_lines_kernel(T* __restrict__ Y, const T* __restrict__ X,
                                                                const T* __restrict__ W,
                                                                const long long* __restrict__ indices, int batch, int h_out,
@@ -160,7 +163,7 @@ __global__ __launch_bounds__(256) void bgmv_expand_lines_kernel(T* __restrict__ 
 #pragma unroll
     for (int q = 0; q < Q; q++) {                     // (rows past the end re-read the last row; their sums are dropped)
       const int row = row0 + q * RPL < h_out ? row0 + q * RPL : h_out - 1;
-      old[q] = yrow[row];
+      old[q] = ACC ? yrow[row] : (T)0;
     }
     if (idx[t] != have) {
       const T* w = W + (idx[t] * num_layers + layer_idx) * (long)h_out * h_in + sub * 8;
@@ -207,6 +210,7 @@ struct SgmvArgsT {
   int n_groups;               // blocks along x: segments, or the maximum length of the tile list
   int n_adapters;
   float scale;
+  int accumulate;             // 1: y += result (the reference's semantics); 0: y = result, y is not read
 };
 
 using SgmvArgs = SgmvArgsT<_Float16>;
@@ -346,7 +350,7 @@ __global__ __launch_bounds__(256) void sgmv_shrink_kernel(const SgmvArgsT<T> a) 
 #pragma unroll
         for (int q = 1; q < R; q++) row = r == q ? rows[q] : row;
         T* yp = a.y + (long)row * a.y_stride + cb2 * 8 + (v2 & 7);
-        *yp = (T)((float)*yp + sum * a.scale);
+        *yp = (T)((a.accumulate ? (float)*yp : 0.f) + sum * a.scale);
       }
     }
   }
@@ -374,7 +378,7 @@ __global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgsT<T> a) 
 #pragma unroll
       for (int i = 0; i < DIN; i++) acc += w[i] * xs[i];
       T* yp = a.y + (long)row * a.y_stride + j;
-      *yp = (T)((float)*yp + acc * a.scale);
+      *yp = (T)((a.accumulate ? (float)*yp : 0.f) + acc * a.scale);
     }
   }
 }
@@ -383,7 +387,7 @@ __global__ __launch_bounds__(256) void sgmv_expand_kernel(const SgmvArgsT<T> a) 
 // A thread owns 8 consecutive output columns: its d_in x 8 weight patch stays in registers while
 // it walks the group's rows R at a time (16-byte loads and stores throughout, no barriers; the R
 // rows' loads are independent, so they are in flight together).
-template <int DIN, int R, class T>
+template <int DIN, int R, class T, bool ACC = true>
 __global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgsT<T> a) {
   SgmvGroupT<T> g;
   if (!sgmv_group(a, blockIdx.x, &g)) return;
@@ -410,7 +414,7 @@ __global__ __launch_bounds__(256) void sgmv_expand_vec_kernel(const SgmvArgsT<T>
 #pragma unroll
       for (int i0 = 0; i0 < DIN / 8; i0++)
         xv[r][i0] = *reinterpret_cast<const lvec8<T>*>(xr + (i0 * 8 < a.d_in ? i0 * 8 : 0));   // same address in every lane
-      old[r] = *reinterpret_cast<const lvec8<T>*>(yp[r]);
+      old[r] = ACC ? *reinterpret_cast<const lvec8<T>*>(yp[r]) : lvec8<T>{0, 0, 0, 0, 0, 0, 0, 0};
     }
     __builtin_amdgcn_sched_barrier(0);   // every request above is issued before the first result is touched
     if (!patch_ready) {

@@ -187,10 +187,21 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
   // routing in its eager form keeps one step in flight (measured: a second step requested ahead of
   // the routing makes the 16-delta case slower, 23.1 against 22.0 us).
   const bool eager = a.raw_indices && a.raw_static;
-  // launches that do not fill the GPU twice over (at most 512 workgroups) are bound by the latency
-  // of each wave's chain of requests rather than by bandwidth: a second step in flight pays there
-  // (5-12 % measured) while it costs time on full launches
-  const bool small = (long)a.n_groups * cb_pad * tsplit * zsplit <= 512;
+  // A launch of at most one live workgroup per CU is bound by the latency of each wave's chain of requests rather
+  // than by bandwidth: a second step in flight pays there, while from two workgroups on some CUs on it costs time
+  // (16 deltas of 4096 x 4096: 8 tokens on 5 deltas, 160 workgroups, 14.6 -> 13.4 us with two steps; 16 tokens on
+  // 11 deltas, 352 workgroups, 18.3 -> 20.3 us; 8192 x 8192: 8 tokens on 6 deltas, 384 workgroups, 31.2 -> 34.0 us;
+  // 11008 x 4096 with 16 tokens on 8 deltas, 256 workgroups, 32.3 -> 29.8 us).  A batch routed inside the kernel
+  // launches a workgroup for every delta that could be in use; the ones that find tokens are estimated as under a
+  // uniform routing, deltas x (1 - (1 - 1 / deltas) ^ tokens).
+  double live_groups = a.n_groups;
+  if (a.raw_indices && !a.raw_static && a.n_deltas > 0) {
+    double none = 1.0;
+    for (int t = 0; t < a.raw_count && none > 1e-9; t++) none *= 1.0 - 1.0 / a.n_deltas;
+    live_groups = a.n_deltas * (1.0 - none);
+    if (live_groups > a.n_groups) live_groups = a.n_groups;
+  }
+  const bool small = live_groups * cb_pad * tsplit * zsplit <= 256.5;
   const int depth = knob_or(knobs().depth, eager || kw == 8 ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1));
   if (eager && !(kw == 4 && ((nt == 1 && depth == 2) || (nt == 1 && depth == 1) || (nt == 2 && depth == 1) || (nt == 4 && depth == 1)))) {
     a.raw_static = 0;   // no eager build of this variant: route first, then request
@@ -258,6 +269,9 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.k = prob_k;
   a.n_deltas = n_deltas;
   a.xcd_swizzle = knobs().xcd_swizzle;
+#ifdef TRITEIA_EXP
+  { const char* e = getenv("XX_PAIR"); a.xx_pair = e ? atoi(e) : 0; e = getenv("XX_A"); a.xx_a = e ? atoi(e) : 0; e = getenv("XX_B"); a.xx_b = e ? atoi(e) : 0; e = getenv("XX_TL_PTR"); a.tl = e ? reinterpret_cast<long long*>(strtoull(e, nullptr, 0)) : nullptr; }
+#endif
 }
 
 
@@ -1015,7 +1029,7 @@ int triteia_hip_sbmm_2_4_routed_static(const void* A, const void* B, const void*
 namespace {
 typedef __bf16 bf16_t;
 
-template <class T>
+template <class T, bool ACC = true>
 int bgmv_impl(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out, int num_layers,
               int layer_idx, float scale, int dev, void* stream) {
   if (batch < 0 || h_in <= 0 || h_out <= 0 || num_layers <= 0 || layer_idx < 0 || layer_idx >= num_layers)
@@ -1029,7 +1043,7 @@ int bgmv_impl(void* Y, const void* X, const void* W, const void* indices, int ba
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (h_in >= h_out) {
-    hipLaunchKernelGGL(bgmv_shrink_kernel<T>, dim3(batch), dim3(256), 0, st, static_cast<T*>(Y), static_cast<const T*>(X),
+    hipLaunchKernelGGL((bgmv_shrink_kernel<T, ACC>), dim3(batch), dim3(256), 0, st, static_cast<T*>(Y), static_cast<const T*>(X),
                        static_cast<const T*>(W), static_cast<const long long*>(indices), h_in, h_out, (long)num_layers,
                        (long)layer_idx, scale);
   } else if (h_in == 8 || h_in == 16 || h_in == 32 || h_in == 64 || h_in == 128) {
@@ -1037,14 +1051,14 @@ int bgmv_impl(void* Y, const void* X, const void* W, const void* indices, int ba
     constexpr int Q = 8, TB = 4;
     const int rows_per_block = 4 * Q * 64 / (h_in / 8);
     const dim3 grid((h_out + rows_per_block - 1) / rows_per_block, (batch + TB - 1) / TB);
-#define BGMV_LINES(LPR_) hipLaunchKernelGGL((bgmv_expand_lines_kernel<T, LPR_, Q, TB>), grid, dim3(256), 0, st, static_cast<T*>(Y), \
+#define BGMV_LINES(LPR_) hipLaunchKernelGGL((bgmv_expand_lines_kernel<T, LPR_, Q, TB, ACC>), grid, dim3(256), 0, st, static_cast<T*>(Y), \
       static_cast<const T*>(X), static_cast<const T*>(W), static_cast<const long long*>(indices), batch, h_out, (long)num_layers, \
       (long)layer_idx, scale)
     if (h_in == 8) BGMV_LINES(1); else if (h_in == 16) BGMV_LINES(2); else if (h_in == 32) BGMV_LINES(4);
     else if (h_in == 64) BGMV_LINES(8); else BGMV_LINES(16);
 #undef BGMV_LINES
   } else {
-    hipLaunchKernelGGL(bgmv_expand_kernel<T>, dim3((h_out + 2047) / 2048, batch), dim3(256), 0, st, static_cast<T*>(Y),
+    hipLaunchKernelGGL((bgmv_expand_kernel<T, ACC>), dim3((h_out + 2047) / 2048, batch), dim3(256), 0, st, static_cast<T*>(Y),
                        static_cast<const T*>(X), static_cast<const T*>(W), static_cast<const long long*>(indices), h_in,
                        h_out, (long)num_layers, (long)layer_idx, scale);
   }
@@ -1079,8 +1093,10 @@ int launch_sgmv(SgmvArgsT<T> a, int max_rows, hipStream_t st) {
     const int rz = row_slots < 8 ? row_slots : 8;
     const dim3 grid(a.n_groups, (a.d_out + 255) / 256, rz);
     const int col_blocks = (a.d_out + 2047) / 2048;
-    if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_vec_kernel<16, kExpandRows16, T>), dim3(a.n_groups, col_blocks, slots(kExpandRows16)), dim3(256), 0, st, a);
-    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_vec_kernel<32, 2, T>), dim3(a.n_groups, col_blocks, slots(2)), dim3(256), 0, st, a);
+    if (a.d_in <= 16 && a.accumulate) hipLaunchKernelGGL((sgmv_expand_vec_kernel<16, kExpandRows16, T, true>), dim3(a.n_groups, col_blocks, slots(kExpandRows16)), dim3(256), 0, st, a);
+    else if (a.d_in <= 16) hipLaunchKernelGGL((sgmv_expand_vec_kernel<16, kExpandRows16, T, false>), dim3(a.n_groups, col_blocks, slots(kExpandRows16)), dim3(256), 0, st, a);
+    else if (a.d_in <= 32 && a.accumulate) hipLaunchKernelGGL((sgmv_expand_vec_kernel<32, 2, T, true>), dim3(a.n_groups, col_blocks, slots(2)), dim3(256), 0, st, a);
+    else if (a.d_in <= 32) hipLaunchKernelGGL((sgmv_expand_vec_kernel<32, 2, T, false>), dim3(a.n_groups, col_blocks, slots(2)), dim3(256), 0, st, a);
     else if (a.d_in <= 64) hipLaunchKernelGGL((sgmv_expand_kernel<64, T>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((sgmv_expand_kernel<128, T>), grid, dim3(256), 0, st, a);
   }
@@ -1089,7 +1105,7 @@ int launch_sgmv(SgmvArgsT<T> a, int max_rows, hipStream_t st) {
 
 template <class T>
 int sgmv_impl(void* y, const void* x, const void* w_ptrs, const void* s, int num_problems, int d_in, int d_out, int layer_idx,
-              int dev, void* stream) {
+              int accumulate, int dev, void* stream) {
   if (num_problems < 0 || d_in <= 0 || d_out <= 0 || layer_idx < 0)
     return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sgmv: problems=%d d_in=%d d_out=%d layer=%d", num_problems, d_in, d_out, layer_idx);
   if (num_problems == 0) return TRITEIA_HIP_OK;
@@ -1110,13 +1126,15 @@ int sgmv_impl(void* y, const void* x, const void* w_ptrs, const void* s, int num
   a.n_groups = num_problems;
   a.n_adapters = num_problems;
   a.scale = 1.0f;
+  a.accumulate = accumulate;
   // segment lengths live on the device; size the row-tile dimension for a few rows per segment
   return launch_sgmv(a, 64, static_cast<hipStream_t>(stream));
 }
 
 template <class T>
 int sgmv_routed_impl(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride, int n_adapters,
-                     int d_in, int d_out, float scale, const void* plan, int prob_n, int dev, void* stream) {
+                     int d_in, int d_out, float scale, const void* plan, int prob_n, int accumulate, int dev, void* stream) {
+  if (accumulate != 0 && accumulate != 1) return fail(TRITEIA_HIP_ERR_ARGUMENT, "sgmv_routed: accumulate=%d", accumulate);
   if (prob_n < 0 || n_adapters < 0 || d_in <= 0 || d_out <= 0)
     return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "sgmv_routed: tokens=%d adapters=%d d_in=%d d_out=%d", prob_n, n_adapters, d_in, d_out);
   if (prob_n == 0 || n_adapters == 0) return TRITEIA_HIP_OK;
@@ -1143,6 +1161,7 @@ int sgmv_routed_impl(void* y, long y_stride, const void* x, long x_stride, const
   a.n_groups = plan_max_tiles(prob_n, n_adapters, triteia_hip_plan_tile_tokens(prob_n, n_adapters));
   a.n_adapters = n_adapters;
   a.scale = scale;
+  a.accumulate = accumulate;
   return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream));
 }
 }  // namespace
@@ -1157,6 +1176,14 @@ int triteia_hip_bgmv_bf16(void* Y, const void* X, const void* W, const void* ind
                           int num_layers, int layer_idx, float scale, int dev, void* stream) {
   return bgmv_impl<bf16_t>(Y, X, W, indices, batch, h_in, h_out, num_layers, layer_idx, scale, dev, stream);
 }
+int triteia_hip_bgmv_store(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                           int num_layers, int layer_idx, float scale, int dev, void* stream) {
+  return bgmv_impl<_Float16, false>(Y, X, W, indices, batch, h_in, h_out, num_layers, layer_idx, scale, dev, stream);
+}
+int triteia_hip_bgmv_store_bf16(void* Y, const void* X, const void* W, const void* indices, int batch, int h_in, int h_out,
+                                int num_layers, int layer_idx, float scale, int dev, void* stream) {
+  return bgmv_impl<bf16_t, false>(Y, X, W, indices, batch, h_in, h_out, num_layers, layer_idx, scale, dev, stream);
+}
 
 size_t triteia_hip_sgmv_tmp_size(int num_problems) {
   // the reference's CUTLASS argument block: 60 bytes per problem (sgmv.cuh:48-52)
@@ -1166,23 +1193,31 @@ size_t triteia_hip_sgmv_tmp_size(int num_problems) {
 int triteia_hip_sgmv(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
                      int d_out, int layer_idx, int dev, void* stream) {
   (void)tmp;
-  return sgmv_impl<_Float16>(y, x, w_ptrs, s, num_problems, d_in, d_out, layer_idx, dev, stream);
+  return sgmv_impl<_Float16>(y, x, w_ptrs, s, num_problems, d_in, d_out, layer_idx, 1, dev, stream);
 }
 int triteia_hip_sgmv_bf16(void* y, const void* x, const void* w_ptrs, const void* s, void* tmp, int num_problems, int d_in,
                           int d_out, int layer_idx, int dev, void* stream) {
   (void)tmp;
-  return sgmv_impl<bf16_t>(y, x, w_ptrs, s, num_problems, d_in, d_out, layer_idx, dev, stream);
+  return sgmv_impl<bf16_t>(y, x, w_ptrs, s, num_problems, d_in, d_out, layer_idx, 1, dev, stream);
+}
+int triteia_hip_sgmv_store(void* y, const void* x, const void* w_ptrs, const void* s, int num_problems, int d_in, int d_out,
+                           int layer_idx, int dev, void* stream) {
+  return sgmv_impl<_Float16>(y, x, w_ptrs, s, num_problems, d_in, d_out, layer_idx, 0, dev, stream);
+}
+int triteia_hip_sgmv_store_bf16(void* y, const void* x, const void* w_ptrs, const void* s, int num_problems, int d_in, int d_out,
+                                int layer_idx, int dev, void* stream) {
+  return sgmv_impl<bf16_t>(y, x, w_ptrs, s, num_problems, d_in, d_out, layer_idx, 0, dev, stream);
 }
 
 int triteia_hip_sgmv_routed(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
                             int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
-                            int dev, void* stream) {
-  return sgmv_routed_impl<_Float16>(y, y_stride, x, x_stride, w_base, w_stride, n_adapters, d_in, d_out, scale, plan, prob_n, dev, stream);
+                            int accumulate, int dev, void* stream) {
+  return sgmv_routed_impl<_Float16>(y, y_stride, x, x_stride, w_base, w_stride, n_adapters, d_in, d_out, scale, plan, prob_n, accumulate, dev, stream);
 }
 int triteia_hip_sgmv_routed_bf16(void* y, long y_stride, const void* x, long x_stride, const void* w_base, long w_stride,
                                  int n_adapters, int d_in, int d_out, float scale, const void* plan, int prob_n,
-                                 int dev, void* stream) {
-  return sgmv_routed_impl<bf16_t>(y, y_stride, x, x_stride, w_base, w_stride, n_adapters, d_in, d_out, scale, plan, prob_n, dev, stream);
+                                 int accumulate, int dev, void* stream) {
+  return sgmv_routed_impl<bf16_t>(y, y_stride, x, x_stride, w_base, w_stride, n_adapters, d_in, d_out, scale, plan, prob_n, accumulate, dev, stream);
 }
 
 }  // extern "C"

@@ -48,9 +48,13 @@ SIGNATURES = {
     "triteia_hip_bgmv_bf16": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_float, _c_int, _c_vp]),
     "triteia_hip_sgmv_bf16": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp]),
     "triteia_hip_sgmv_routed_bf16": (_c_int, [_c_vp, _c_long, _c_vp, _c_long, _c_vp, _c_long] + [_c_int] * 3
-                                     + [_c_float, _c_vp, _c_int, _c_int, _c_vp]),
+                                     + [_c_float, _c_vp, _c_int, _c_int, _c_int, _c_vp]),
     "triteia_hip_sgmv_routed": (_c_int, [_c_vp, _c_long, _c_vp, _c_long, _c_vp, _c_long] + [_c_int] * 3
-                                + [_c_float, _c_vp, _c_int, _c_int, _c_vp]),
+                                + [_c_float, _c_vp, _c_int, _c_int, _c_int, _c_vp]),
+    "triteia_hip_bgmv_store": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_float, _c_int, _c_vp]),
+    "triteia_hip_bgmv_store_bf16": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_float, _c_int, _c_vp]),
+    "triteia_hip_sgmv_store": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_vp]),
+    "triteia_hip_sgmv_store_bf16": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_vp]),
 }
 
 _lib = None

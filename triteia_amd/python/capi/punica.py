@@ -24,9 +24,10 @@ def _check(err):
         raise RuntimeError(f"triteia_hip error {err}: {_ffi.last_error()}")
 
 
-def sgmv(y, x, w_ptr, s, tmp, layer_idx):
+def sgmv(y, x, w_ptr, s, tmp, layer_idx, accumulate=True):
     """y[s[i]:s[i+1]] += x[s[i]:s[i+1]] @ deref(w_ptr[i])[layer_idx]
-    (the reference's `sgmv_cutlass` binding, triteia/csrc/ops/ops.cpp:120-147)."""
+    (the reference's `sgmv_cutlass` binding, triteia/csrc/ops/ops.cpp:120-147).
+    `accumulate=False` (no counterpart in the reference) stores the product instead of adding it: y is not read."""
     _ffi.require_gpu(y=y, x=x, w_ptr=w_ptr, s=s, tmp=tmp)
     if y.dim() != 2 or x.dim() != 2 or w_ptr.dim() != 1 or s.dim() != 1 or tmp.dim() != 1:
         raise RuntimeError("y, x must be 2D tensors; w_ptr, s, tmp 1D tensors")
@@ -39,6 +40,11 @@ def sgmv(y, x, w_ptr, s, tmp, layer_idx):
     if tmp.numel() * tmp.element_size() != sgmv_tmp_size(num_problems):
         raise RuntimeError(f"CHECK_EQ(tmp.size(0), sgmv_tmp_size(num_problems)) failed. "
                            f"{tmp.numel()} vs {sgmv_tmp_size(num_problems)}")
+    if not accumulate:
+        fn = _ffi.lib().triteia_hip_sgmv_store if dtype == torch.float16 else _ffi.lib().triteia_hip_sgmv_store_bf16
+        _check(fn(_ffi.ptr(y), _ffi.ptr(x), _ffi.ptr(w_ptr), _ffi.ptr(s), num_problems, x.size(1), y.size(1),
+                  int(layer_idx), _ffi.device_index(x), _ffi.stream_of(x)))
+        return
     fn = _ffi.lib().triteia_hip_sgmv if dtype == torch.float16 else _ffi.lib().triteia_hip_sgmv_bf16
     _check(fn(
         _ffi.ptr(y), _ffi.ptr(x), _ffi.ptr(w_ptr), _ffi.ptr(s), _ffi.ptr(tmp), num_problems, x.size(1), y.size(1),
@@ -49,8 +55,9 @@ def sgmv_tmp_size(num_problems):
     return _ffi.lib().triteia_hip_sgmv_tmp_size(int(num_problems))
 
 
-def dispatch_bgmv(y, x, w, indicies, layer_idx, scale):
-    """y[b] += scale * w[indicies[b], layer_idx] @ x[b]  (triteia/csrc/ops/ops.cpp:177-220)."""
+def dispatch_bgmv(y, x, w, indicies, layer_idx, scale, accumulate=True):
+    """y[b] += scale * w[indicies[b], layer_idx] @ x[b]  (triteia/csrc/ops/ops.cpp:177-220).
+    `accumulate=False` (no counterpart in the reference) stores the product instead of adding it: y is not read."""
     _ffi.require_gpu(y=y, x=x, w=w, indicies=indicies)
     if y.dim() != 2 or x.dim() != 2 or w.dim() != 4 or indicies.dim() != 1:
         raise RuntimeError("y, x must be 2D tensors, w a 4D tensor, indicies a 1D tensor")
@@ -62,7 +69,10 @@ def dispatch_bgmv(y, x, w, indicies, layer_idx, scale):
                        (indicies.size(0), B, "indicies.size(0), x.size(0)"), (y.size(0), B, "y.size(0), x.size(0)")):
         if a != b:
             raise RuntimeError(f"CHECK_EQ({what}) failed. {a} vs {b}")
-    fn = _ffi.lib().triteia_hip_bgmv if dtype == torch.float16 else _ffi.lib().triteia_hip_bgmv_bf16
+    if accumulate:
+        fn = _ffi.lib().triteia_hip_bgmv if dtype == torch.float16 else _ffi.lib().triteia_hip_bgmv_bf16
+    else:
+        fn = _ffi.lib().triteia_hip_bgmv_store if dtype == torch.float16 else _ffi.lib().triteia_hip_bgmv_store_bf16
     _check(fn(
         _ffi.ptr(y), _ffi.ptr(x), _ffi.ptr(w), _ffi.ptr(indicies), B, h_in, h_out, w.size(1), int(layer_idx),
         float(scale), _ffi.device_index(x), _ffi.stream_of(x)))
@@ -75,8 +85,9 @@ def add_lora_sgmv_cutlass(y, x, wa_ptr, wb_ptr, s, layer_idx, lora_rank):
     [num_layers, H1, R] / [num_layers, R, H2] fp16 matrices, s int32 [S+1] indptr."""
     tmp_size = sgmv_tmp_size(wa_ptr.size(0))
     tmp = torch.empty((tmp_size,), dtype=torch.uint8, device=x.device)
-    v = torch.zeros((x.size(0), lora_rank), dtype=x.dtype, device=x.device)
-    sgmv(v, x, wa_ptr, s, tmp, layer_idx)
+    # the shrink stores its result: the intermediate needs no clearing, and only rows inside a segment are read back
+    v = torch.empty((x.size(0), lora_rank), dtype=x.dtype, device=x.device)
+    sgmv(v, x, wa_ptr, s, tmp, layer_idx, accumulate=False)
     sgmv(y, v, wb_ptr, s, tmp, layer_idx)
 
 
@@ -86,13 +97,15 @@ def add_lora_bgmv(y, x, wa_T_all, wb_T_all, indicies, layer_idx, scale):
     y [B, H2] (changed in place), x [B, H1], wa_T_all [n, L, R, H1], wb_T_all [n, L, H2, R],
     indicies int64 [B]."""
     r = wb_T_all.size(-1)
-    tmp = torch.zeros((x.size(0), r), dtype=x.dtype, device=x.device)
-    dispatch_bgmv(tmp, x, wa_T_all, indicies, layer_idx, 1.0)
+    # the shrink stores its result: the intermediate needs no clearing (rows with a negative index are never read back)
+    tmp = torch.empty((x.size(0), r), dtype=x.dtype, device=x.device)
+    dispatch_bgmv(tmp, x, wa_T_all, indicies, layer_idx, 1.0, accumulate=False)
     dispatch_bgmv(y, tmp, wb_T_all, indicies, layer_idx, scale)
 
 
-def sgmv_routed(y, x, weights, plan, scale=1.0):
-    """y[t] += scale * x[t] @ weights[a] for every token t the routing plan lists under adapter a.
+def sgmv_routed(y, x, weights, plan, scale=1.0, accumulate=True):
+    """y[t] += scale * x[t] @ weights[a] for every token t the routing plan lists under adapter a
+    (`accumulate=False`: stored instead of added; y is not read, rows the plan does not list keep what they hold).
 
     weights [n_adapters, d_in, d_out] fp16 or bf16 (as x and y), contiguous; `plan` from capi.route_plan with
     n_deltas == n_adapters."""
@@ -104,4 +117,4 @@ def sgmv_routed(y, x, weights, plan, scale=1.0):
     fn = _ffi.lib().triteia_hip_sgmv_routed if dtype == torch.float16 else _ffi.lib().triteia_hip_sgmv_routed_bf16
     _check(fn(
         _ffi.ptr(y), y.stride(0), _ffi.ptr(x), x.stride(0), _ffi.ptr(weights), d_in * d_out, n_adapters, d_in, d_out,
-        float(scale), _ffi.ptr(plan), x.size(0), _ffi.device_index(x), _ffi.stream_of(x)))
+        float(scale), _ffi.ptr(plan), x.size(0), 1 if accumulate else 0, _ffi.device_index(x), _ffi.stream_of(x)))

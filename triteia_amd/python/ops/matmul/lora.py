@@ -60,7 +60,7 @@ def lora_sgmv_routed(weights_A, weights_B, x, indices, base_weight=None, plan=No
     if plan is None:
         plan = route_plan(indices.to(torch.int32), n_adapters)
     x = x if x.is_contiguous() else x.contiguous()
-    v = torch.zeros((x.shape[0], rank), dtype=x.dtype, device=x.device)
-    sgmv_routed(v, x, weights_A.contiguous(), plan)
+    v = torch.empty((x.shape[0], rank), dtype=x.dtype, device=x.device)
+    sgmv_routed(v, x, weights_A.contiguous(), plan, accumulate=False)    # (the expand reads back routed rows only)
     sgmv_routed(y, v, weights_B.contiguous(), plan)
     return y
