@@ -113,11 +113,6 @@ struct Sparse24Args {
   // 1: the plan's tiles hold up to 64 tokens and the 32-token build of the wide kernel takes each as two halves
   // (workgroups 2g and 2g + 1 of a column group; a half without tokens returns at once)
   int tile_halves;
-#ifdef TRITEIA_EXP
-  int xx_pair;      // experiment: units u and u + gridDim.x / 2 take adjacent column blocks of one group
-  int xx_a, xx_b;
-  long long* tl;    // timeline marks: [workgroup][8 waves][8 events]
-#endif
 };
 
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
@@ -163,21 +158,6 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-#if defined(TRITEIA_EXP_TL)
-__device__ __forceinline__ void tl_mark(const Sparse24Args& p, int ev) {
-  if (p.tl && (threadIdx.x & 63) == 0) {
-    const long w = ((long)blockIdx.x * 8 + (threadIdx.x >> 6));
-    long long v = (long long)wall_clock64();
-    if (ev == 7) v = (long long)__builtin_amdgcn_s_getreg(63492) | ((long long)__builtin_amdgcn_s_getreg(63508) << 32);
-    p.tl[w * 8 + ev] = v;
-  }
-}
-#define TL_MARK(p, ev) tl_mark(p, ev)
-#define TL_MARK_AFTER(p, ev, reg) do { asm volatile("" :: "v"(reg)); tl_mark(p, ev); } while (0)
-#else
-#define TL_MARK(p, ev)
-#define TL_MARK_AFTER(p, ev, reg)
-#endif
 template <int NT>
 struct StepFrag {
   uint4_t wq[4];        // weights: groups a and a+4 (a = vector index) of 8 columns
@@ -370,46 +350,18 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   // registers (ring of fragments, statically indexed through the unrolled inner loop).
   // The body is branch-free apart from the wave-uniform "is this step real" test around the
   // arithmetic, so each iteration issues the same loads and waits for exactly its own.
-#if defined(TRITEIA_EXP_DB)
-  if constexpr (DEPTH == 1) {
-    // one step in flight at all times: the next step is requested the moment the current one has landed, ahead of
-    // the current step's arithmetic
-    StepFrag<NTT> alt;
-    load_x(ring[0], wave);
-    for (int st = wave; st < n_steps; st += 2 * KW) {
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __builtin_amdgcn_sched_barrier(0);
-      load_w(alt, st + KW);
-      load_x(alt, st + KW);
-      __builtin_amdgcn_sched_barrier(0);
-      compute_step(ring[0], st);
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __builtin_amdgcn_sched_barrier(0);
-      load_w(ring[0], st + 2 * KW);
-      load_x(ring[0], st + 2 * KW);
-      __builtin_amdgcn_sched_barrier(0);
-      if (st + KW < n_steps) compute_step(alt, st + KW);
-    }
-  } else
-#endif
-  {
 #pragma unroll
   for (int j = 0; j < DEPTH; j++) load_x(ring[j], wave + j * KW);
-  TL_MARK(p, 2);
   for (int st = wave; st < n_steps; st += DEPTH * KW) {
 #pragma unroll
     for (int j = 0; j < DEPTH; j++) {
       const int cur = st + j * KW;
       if (cur < n_steps) compute_step(ring[j], cur);
-      if (st == wave && j == 0) TL_MARK_AFTER(p, 3, acc[0][0][0]);
-      if (st == wave + DEPTH * KW && j == 0) TL_MARK_AFTER(p, 6, acc[0][0][0]);
       load_w(ring[j], cur + DEPTH * KW);
       load_x(ring[j], cur + DEPTH * KW);
     }
   }
-  }
 
-  TL_MARK_AFTER(p, 4, acc[0][0][0]);
   // cross-wave reduction + epilogue, one 16-token tile at a time
 #pragma unroll
   for (int nt = 0; nt < NTT; nt++) {
@@ -459,7 +411,6 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
       *reinterpret_cast<half8_t*>(op) = o;
     }
   }
-  TL_MARK(p, 5);
 }
 
 // NT = widest token tile (16*NT tokens per pass) the instantiation supports; narrower passes
@@ -467,12 +418,7 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 // EAGER: fused routing with group g = delta g (Sparse24Args::raw_static): the weights of the first
 // step are requested at once, together with the indices, instead of one memory round trip later.
 template <int NT, int KW, int DEPTH, bool EAGER = false>
-#if defined(TRITEIA_EXP_DB)
-#define TRITEIA_NT1_D1_WGS 2
-#else
-#define TRITEIA_NT1_D1_WGS 3
-#endif
-__global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? TRITEIA_NT1_D1_WGS : 2) : (NT == 2 ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
+__global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2 ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
   // steps per wave requested ahead of the routing in the EAGER build (the 32- and 64-token builds
   // also hold narrower passes with a ring of their own depth: one step fits them all)
   constexpr int NPRE = EAGER ? (NT == 1 ? DEPTH : 1) : 0;
@@ -485,35 +431,13 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? TRITEIA_NT1_D1_WG
   // (with sub_shift > 0 the same holds for the shares of column blocks)
   const int col_units = (p.m >> 7) << p.sub_shift;
   const int cu_pad = (col_units + 7) & ~7;
-  int unit = blockIdx.x;
-#ifdef TRITEIA_EXP
-  if (p.xx_pair && (gridDim.x & 1) == 0) {
-    const int half = gridDim.x >> 1;
-    const int u2 = unit >= half ? unit - half : unit;
-    unit = 2 * u2 + (blockIdx.x >= half ? 1 : 0);
-  }
-#endif
+  const int unit = blockIdx.x;
   const int grp = unit / cu_pad;
   const int i = unit - grp * cu_pad;
-#ifdef TRITEIA_EXP
-  // with pairing, unit v = 2 u2 + p runs on XCD u2 % 8 = (i >> 1) % 8: XCD x takes column blocks {(cu_pad / 8) x ..}
-  const int cu0 = p.xx_pair ? (p.xcd_swizzle ? ((i >> 1) & 7) * (cu_pad >> 3) + ((i >> 4) << 1) + (i & 1) : i)
-                           : (p.xcd_swizzle ? (i & 7) * (cu_pad >> 3) + (i >> 3) : i);
-#else
-  const int cu0 = p.xcd_swizzle ? (i & 7) * (cu_pad >> 3) + (i >> 3) : i;
-#endif
-  if (cu0 >= col_units) return;
-#ifdef TRITEIA_EXP
-  // experiment: the column units of group g are rotated by xx_a * g, so that an XCD's requests are spread over every
-  // position inside a packed row instead of the same 1/8 of each row for all deltas
-  const int cu = p.xx_a ? (cu0 + p.xx_a * grp) % col_units : cu0;
-#else
-  const int cu = cu0;
-#endif
+  const int cu = p.xcd_swizzle ? (i & 7) * (cu_pad >> 3) + (i >> 3) : i;
+  if (cu >= col_units) return;
   const int cb = cu >> p.sub_shift;
 
-  TL_MARK(p, 0);
-  TL_MARK(p, 7);
   TileCtx c;
   c.tid = threadIdx.x;
   c.wave = c.tid >> 6;
@@ -631,7 +555,6 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? TRITEIA_NT1_D1_WG
       count += cj;
     }
     c.raw_before[kRawParts] = count;
-    TL_MARK(p, 1);
     if (EAGER && count <= 0) {
       __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): let the requested weights land before the wave ends
       return;

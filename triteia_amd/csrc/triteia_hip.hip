@@ -269,9 +269,6 @@ void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* met
   a.k = prob_k;
   a.n_deltas = n_deltas;
   a.xcd_swizzle = knobs().xcd_swizzle;
-#ifdef TRITEIA_EXP
-  { const char* e = getenv("XX_PAIR"); a.xx_pair = e ? atoi(e) : 0; e = getenv("XX_A"); a.xx_a = e ? atoi(e) : 0; e = getenv("XX_B"); a.xx_b = e ? atoi(e) : 0; e = getenv("XX_TL_PTR"); a.tl = e ? reinterpret_cast<long long*>(strtoull(e, nullptr, 0)) : nullptr; }
-#endif
 }
 
 
