@@ -859,17 +859,67 @@ def test_lora_ops(ops, T, M, k, m, r, seed):
     check_close(ops.lora_sgmv_routed(gA, gB, gx2, gi2), ref2, what="lora_sgmv_routed unsorted")
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("T,M,k,m,r,seed", [
+    (128, 2, 4096, 12288, 64, 181),      # tests/ops/test_lora_bgmv.py:74
+    (300, 3, 1024, 2048, 32, 182), (70, 2, 512, 520, 128, 183), (41, 5, 768, 256, 64, 184), (200, 4, 1024, 1000, 32, 185),
+    (10, 5, 768, 768, 64, 186),          # short segments through the same kernels
+    (97, 3, 2048, 384, 16, 187),         # rank 16: the shrink only
+])
+def test_lora_on_the_matrix_cores(ops, monkeypatch, T, M, k, m, r, seed, dtype):
+    """SGMV and routed SGMV with every launch the matrix-core kernels can take sent to them (by default: ranks 32 / 64 /
+    128 with 16 rows per group and more), against the oracle; in bf16 with the oracle's bf16 intermediate.  The same
+    calls with those kernels switched off agree to the rounding of the intermediate."""
+    say(f"lora mfma T={T} M={M} k={k} m={m} r={r} seed={seed} {dtype}")
+    rng = np.random.default_rng(seed)
+    idx = np.sort(rng.integers(-1, M, size=T)).astype(np.int32)
+    if dtype == "f16":
+        A, B = _lora_weights(M, k, r, m, seed, scale=0.1)
+        x = activations(T, k, seed + 1)
+        ref = orc.lora(A, B, x, idx)
+        gA, gB, gx = to_gpu(A, B, x)
+        tol = 2e-3
+    else:
+        A = orc.round_bf16(rng.standard_normal((M, k, r)) * 0.1).astype(np.float32)
+        B = orc.round_bf16(rng.standard_normal((M, r, m)) * 0.1).astype(np.float32)
+        x = orc.round_bf16(rng.standard_normal((T, k))).astype(np.float32)
+        ref = orc.lora(A, B, x, idx, intermediate="bf16")
+        gA, gB, gx = (torch.from_numpy(a).to(DEV).to(torch.bfloat16) for a in (A, B, x))
+        tol = 1e-2
+    gi = torch.from_numpy(idx).to(DEV)
+    outs = {}
+    for mode in ("2", "0"):
+        setknob(monkeypatch, "TRITEIA_HIP_LORA_MFMA", mode)
+        for name in ("lora_sgmv", "lora_sgmv_routed"):
+            out = getattr(ops, name)(gA, gB, gx, gi)
+            torch.cuda.synchronize()
+            check_close(out, ref, tol=tol, what=f"{name} (LORA_MFMA={mode})")
+            assert bool((out[torch.from_numpy(idx < 0).to(DEV)] == 0).all())
+            outs[(name, mode)] = out
+    for name in ("lora_sgmv", "lora_sgmv_routed"):
+        d = (outs[(name, "2")].float() - outs[(name, "0")].float()).norm() / outs[(name, "0")].float().norm()
+        assert float(d) < tol, f"{name}: matrix-core and VALU kernels differ by {float(d):.2e}"
+    # unsorted indices through the routed form
+    setknob(monkeypatch, "TRITEIA_HIP_LORA_MFMA", "2")
+    perm = rng.permutation(T)
+    gi2 = torch.from_numpy(idx[perm].copy()).to(DEV)
+    gx2 = gx[torch.from_numpy(perm).to(DEV)].contiguous()
+    check_close(ops.lora_sgmv_routed(gA, gB, gx2, gi2), ref[perm], tol=tol, what="lora_sgmv_routed unsorted (matrix cores)")
+
+
 @pytest.mark.parametrize("T,M,d_in,d_out,seed", [
     (37, 4, 1024, 16, 171), (37, 4, 16, 1024, 172), (90, 3, 512, 64, 173), (90, 3, 64, 520, 174), (20, 2, 768, 128, 175),
     (64, 5, 32, 2048, 176), (50, 3, 24, 256, 177),
 ])
-def test_lora_kernels_store_instead_of_add(T, M, d_in, d_out, seed):
+@pytest.mark.parametrize("mfma", ["0", "2"])
+def test_lora_kernels_store_instead_of_add(monkeypatch, T, M, d_in, d_out, seed, mfma):
     """The stored form of BGMV / SGMV / routed SGMV (no counterpart in the reference; the intermediate of a LoRA pair then
     needs no clearing): rows that take an adapter hold the product alone, whatever the output held before; the others
     keep what they held.  Both directions (wide -> narrow, narrow -> wide), against a plain fp32 product."""
     from triteia_amd.python.capi import route_plan, sgmv_routed
     from triteia_amd.python.capi.punica import dispatch_bgmv, sgmv, sgmv_tmp_size
-    say(f"lora store T={T} M={M} d_in={d_in} d_out={d_out} seed={seed}")
+    say(f"lora store T={T} M={M} d_in={d_in} d_out={d_out} seed={seed} LORA_MFMA={mfma}")
+    setknob(monkeypatch, "TRITEIA_HIP_LORA_MFMA", mfma)
     rng = np.random.default_rng(seed)
     W = (rng.standard_normal((M, d_in, d_out)) * 0.1).astype(np.float16)
     x = (rng.standard_normal((T, d_in))).astype(np.float16)

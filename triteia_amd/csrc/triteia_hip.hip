@@ -11,6 +11,7 @@
 #include <mutex>
 
 #include "lora.hip.h"
+#include "lora_mfma.hip.h"
 #include "route_plan.hip.h"
 #include "sparse24_gemm.hip.h"
 #include "sparse24_share.hip.h"
@@ -58,7 +59,7 @@ struct Knobs {
   int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, wide_order_min_idle = kUnset, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
-  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1;
+  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1, mid_ks64 = 0, lora_mfma = 1;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
   int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset, share16 = 1, share16_max_blocks = kUnset;
 };
@@ -74,7 +75,7 @@ void read_knobs() {
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
       {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
-      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"PLAN_BIG", &k.plan_big}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
+      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"PLAN_BIG", &k.plan_big}, {"MID_KS64", &k.mid_ks64}, {"LORA_MFMA", &k.lora_mfma}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
       {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
       {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift}, {"SHARE16", &k.share16}, {"SHARE16_MAX_BLOCKS", &k.share16_max_blocks},
   };
@@ -905,6 +906,19 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     const int forced = knobs().pass_nt;
     if ((forced == 1 || forced == 2 || forced == 4) && 16 * forced <= tile) pass_nt = forced;
   }
+  // A plan that also lists its tokens in 64-token tiles, on a layer where even the host's bound on those tiles makes at
+  // most one workgroup per CU: the 64-token build on eight wavefronts (K halved inside the workgroup) takes that list.
+  if (knobs().mid_ks64 && plan_has_big(prob_n, n_deltas) && prob_k % 128 == 0 && (long)prob_n * prob_k * 2 < (1L << 32) &&
+      (long)L.max_big * (((prob_m / 128 + 3) / 4 + 7) / 8 * 8) <= knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits)) {
+    a.xcd_swizzle = wide_unit_order(prob_m);
+    a.tiles = reinterpret_cast<const int4*>(ws + L.big);
+    a.tiles_alt = nullptr;
+    a.n_groups_dev = ws + L.header + 6;
+    a.n_groups = L.max_big;
+    hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true, 2>), dim3((unsigned)wide_grid_units(a.n_groups, prob_m, a.xcd_swizzle)), dim3(512), 0,
+                       static_cast<hipStream_t>(stream), a);
+    return check_launch("sparse24_wide_kernel (plan's 64-token tiles, eight wavefronts)");
+  }
   if (mid) a.xcd_swizzle = wide_unit_order(prob_m);
   if (mid && mid_big(prob_n, n_deltas, prob_m, prob_k)) {
     // the plan's own list of 64-token tiles, whole, on the 64-token build
@@ -1071,12 +1085,43 @@ int bgmv_impl(void* Y, const void* X, const void* W, const void* indices, int ba
 constexpr int kShrinkRows16 = TRITEIA_SHRINK_ROWS16;   // token rows a block of the rank <= 16 shrink kernel takes at a time
 constexpr int kExpandRows16 = TRITEIA_EXPAND_ROWS16;
 
+// Adapters of rank 32, 64 or 128 run on the matrix cores (lora_mfma.hip.h): the expand always (512 tokens over 8
+// adapters of rank 64 on 4096 columns 42.9 -> 7.5 us, 256 over 32 on 11008 columns 291 -> 15 us); the shrink, where a
+// workgroup pulls the whole adapter through one CU per pass of tokens, from 128 rows per group on (`rows_per_group`:
+// what the caller knows of the average, 0 = nothing; 2048 tokens over 4 adapters of rank 64 / 128 on k = 4096 46.4 -> 28.9 /
+// 81.1 -> 32.5 us, 512 over 8 20.0 -> 23.2 us).  The knob lora_mfma = 2 sends every launch there that the kernels can
+// take (the shrink also at rank 16), 0 none.
+constexpr int kLoraMfmaShrinkMinRows = 128;
 template <class T>
-int launch_sgmv(SgmvArgsT<T> a, int max_rows, hipStream_t st) {
+bool launch_sgmv_mfma(const SgmvArgsT<T>& a, int max_rows, int rows_per_group, hipStream_t st) {
+  const int mode = knobs().lora_mfma;
+  if (mode == 0) return false;
+  int row_slots = max_rows < 1 ? 1 : max_rows;
+  if (a.d_in >= a.d_out) {
+    if (mode == 1 && rows_per_group < kLoraMfmaShrinkMinRows) return false;
+    if (a.d_in % 32 != 0 || !(a.d_out == 32 || a.d_out == 64 || a.d_out == 128 || (a.d_out == 16 && mode == 2))) return false;
+    if (row_slots > 256) row_slots = 256;
+#define SHRINK_MFMA(R16_, TT_) hipLaunchKernelGGL((sgmv_shrink_mfma_kernel<T, R16_, TT_>), dim3(a.n_groups, (row_slots + 16 * TT_ - 1) / (16 * TT_)), dim3(256), 0, st, a)
+    if (a.d_out == 16) SHRINK_MFMA(1, 4); else if (a.d_out == 32) SHRINK_MFMA(2, 4); else if (a.d_out == 64) SHRINK_MFMA(4, 4); else SHRINK_MFMA(8, 2);
+#undef SHRINK_MFMA
+    return true;
+  }
+  if (!(a.d_in == 32 || a.d_in == 64 || a.d_in == 128)) return false;
+  if (row_slots > 64) row_slots = 64;
+  const dim3 grid(a.n_groups, (a.d_out + 127) / 128, (row_slots + 15) / 16);
+  if (a.d_in == 32) hipLaunchKernelGGL((sgmv_expand_mfma_kernel<T, 1>), grid, dim3(256), 0, st, a);
+  else if (a.d_in == 64) hipLaunchKernelGGL((sgmv_expand_mfma_kernel<T, 2>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((sgmv_expand_mfma_kernel<T, 4>), grid, dim3(256), 0, st, a);
+  return true;
+}
+
+template <class T>
+int launch_sgmv(SgmvArgsT<T> a, int max_rows, hipStream_t st, int rows_per_group = 0) {
   const int narrow = a.d_in < a.d_out ? a.d_in : a.d_out;
   if (a.d_in % 8 != 0 || a.d_out % 8 != 0 || narrow > kLoraMaxNarrow)
     return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "No suitable kernel. d_in=%d d_out=%d", a.d_in, a.d_out);
   if (a.n_groups <= 0) return TRITEIA_HIP_OK;
+  if (launch_sgmv_mfma(a, max_rows, rows_per_group, st)) return check_launch("sgmv kernel (matrix cores)");
   // rows of a group are spread over y (shrink) / z (expand); group sizes live on the device
   int row_slots = max_rows < 64 ? max_rows : 64;
   if (row_slots < 1) row_slots = 1;
@@ -1159,7 +1204,7 @@ int sgmv_routed_impl(void* y, long y_stride, const void* x, long x_stride, const
   a.n_adapters = n_adapters;
   a.scale = scale;
   a.accumulate = accumulate;
-  return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream));
+  return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream), prob_n / (n_adapters < prob_n ? n_adapters : prob_n));
 }
 }  // namespace
 
