@@ -202,10 +202,13 @@ TRITEIA_HIP_API int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, in
 /* The order in which sparse24_wide_kernel numbers its units (token tile x group of 512 columns) on a layer of prob_m
  * columns (1: column groups padded to a multiple of 8, a contiguous run per XCD; 3: the same with the padding's idle
  * slots put to work, on layers where the padding would leave XCDs short of work; 0 / 2 by environment only), and the
- * number of workgroups of a launch over `rows` tiles in a given order.  No counterpart in the reference; for the tests
+ * number of workgroups of a launch over `rows` tiles in a given order; for the order that the host picks per launch
+ * (4: every XCD takes a block of `block_column_groups` column groups x a block of tiles), the number of workgroups
+ * by block size, -1 where the layer's padded column groups cannot be cut that way over 8 XCDs.  No counterpart in the reference; for the tests
  * that check each order against a restatement of the kernel's index arithmetic. */
 TRITEIA_HIP_API int triteia_hip_wide_unit_order(int prob_m);
 TRITEIA_HIP_API long triteia_hip_wide_grid_units(long rows, int prob_m, int order);
+TRITEIA_HIP_API long triteia_hip_wide_block_grid_units(long rows, int prob_m, int block_column_groups);
 
 /* 1 or 2 if triteia_hip_sbmm_2_4_routed handles this batch and layer in one launch, routing inside the multiply kernel
  * (the workspace stays untouched; 2: at most 16 tokens on the column-share kernel, sparse24_share16_kernel, 1: the

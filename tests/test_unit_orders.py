@@ -34,6 +34,48 @@ def unit_of(u, cgs, rows, order):
     return grp, cg
 
 
+def block_unit_of(u, cgs, rows_live, xc):
+    """Order 4: XCD u % 8 takes block (u % 8) % n of the column groups and block (u % 8) // n of the live tiles."""
+    cg_pad = (cgs + 7) // 8 * 8
+    n_cgb = cg_pad // xc
+    tbs = 8 // n_cgb
+    tpb = (rows_live + tbs - 1) // tbs
+    xcd, slot = u & 7, u >> 3
+    cg = (xcd % n_cgb) * xc + slot % xc
+    tslot = slot // xc
+    grp = (xcd // n_cgb) * tpb + tslot
+    if tslot >= tpb or grp >= rows_live or cg >= cgs:
+        return None
+    return grp, cg
+
+
+def test_blocks_per_xcd_give_every_unit_once():
+    """The grid is sized on the host's bound of tiles; the device cuts the blocks of tiles from the live count."""
+    lib = _ffi.lib()
+    for cgs in range(1, 41):
+        cg_pad = (cgs + 7) // 8 * 8
+        m = 512 * cgs
+        sizes = [xc for xc in range(1, cg_pad + 1) if cg_pad % xc == 0 and cg_pad // xc <= 8 and 8 % (cg_pad // xc) == 0]
+        assert cg_pad // 8 in sizes and cg_pad in sizes
+        for xc in range(1, cg_pad + 1):
+            if xc not in sizes:
+                assert lib.triteia_hip_wide_block_grid_units(5, m, xc) == -1
+        for xc in sizes:
+            for rows in list(range(1, 20)) + [127, 129, 500]:
+                grid = lib.triteia_hip_wide_block_grid_units(rows, m, xc)
+                assert grid > 0 and grid % 8 == 0
+                for rows_live in {rows, max(1, rows // 2), max(1, rows - 1), 1}:
+                    seen = collections.Counter()
+                    per_xcd = collections.defaultdict(set)
+                    for u in range(grid):
+                        t = block_unit_of(u, cgs, rows_live, xc)
+                        if t is not None:
+                            seen[t] += 1
+                            per_xcd[u % 8].add(t[1])
+                    assert len(seen) == rows_live * cgs and set(seen.values()) == {1}, (cgs, xc, rows, rows_live)
+                    assert all(len(v) <= xc for v in per_xcd.values())
+
+
 @pytest.mark.parametrize("order", [0, 1, 2, 3])
 def test_every_unit_once_and_none_past_the_bound(order):
     lib = _ffi.lib()

@@ -99,6 +99,7 @@ struct Sparse24Args {
   int raw_static;           // fused routing with group g = delta g: weights are requested before the indices arrive
   int rot_spread;           // steps between the starting points of consecutive deltas' walks over K (0: all start at step 0)
   int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run
+  int xcd_cgs;              // wide kernel, order 4: column groups (of 512) in the block that one XCD takes
   // K split across workgroups (uniform groups only): blockIdx.z = z takes the steps [z * ksplit_steps, (z + 1) * ksplit_steps)
   // of K and writes its fp32 sums, unscaled, to partial[z][row][column]; splitk_reduce_kernel adds the splits in
   // the order of z and finishes the rows.  ksplit_steps = 0: no split.

@@ -80,6 +80,24 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
       cg = row * pad + (c - cgs);
     }
     if (grp >= rows_of_tiles) return;
+  } else if (p.xcd_swizzle == 4) {
+    // an XCD takes a block of xcd_cgs column groups x a block of tiles: the bytes that its L2 has to fetch are the
+    // block's weights plus the block's activations, least when the two are of about the same size
+    // (a plan's list: the blocks of tiles are cut from the list's real length, which the device knows, so that the
+    // live tiles spread over all the XCDs; the launch is sized for the host's bound on it)
+    int rows_live = rows_of_tiles;
+    if (p.tiles && p.n_groups_dev) {
+      const bool alt = PLAN_ALL && p.tiles_alt && (long)p.n_groups_dev[4] * p.wide_gate < p.wide_min_units;
+      rows_live = min(rows_of_tiles, p.n_groups_dev[alt ? 5 : 0] * (PLAN_ALL && TOK == 32 && p.tile_halves ? 2 : 1));
+    }
+    const int n_cgb = cg_pad / p.xcd_cgs;             // blocks of column groups (a divisor of 8)
+    const int tbs = 8 / n_cgb;                         // blocks of tiles
+    const int tpb = (rows_live + tbs - 1) / tbs;       // tiles per block
+    const int xcd = unit & 7, slot = unit >> 3;
+    cg = (xcd % n_cgb) * p.xcd_cgs + slot % p.xcd_cgs;
+    const int tslot = slot / p.xcd_cgs;
+    grp = (xcd / n_cgb) * tpb + tslot;
+    if (tslot >= tpb || grp >= rows_live) return;
   } else {
     cg = p.xcd_swizzle ? (i & 7) * (cg_pad >> 3) + (i >> 3) : i;
   }

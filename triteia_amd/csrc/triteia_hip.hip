@@ -56,10 +56,10 @@ int check_launch(const char* what) {
 // kUnset marks knobs whose default depends on the launch.
 constexpr int kUnset = -0x7fffffff;
 struct Knobs {
-  int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, wide_order_min_idle = kUnset, pass_nt = 0;
+  int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, xcd_cgs = 0 /* 0: the rule, n > 0: blocks of n column groups, -1: never */, wide_order_min_idle = kUnset, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
-  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1, mid_ks64 = 0, lora_mfma = 1;
+  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1, lora_mfma = 1;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
   int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset, share16 = 1, share16_max_blocks = kUnset;
 };
@@ -69,13 +69,13 @@ std::once_flag g_knobs_once;
 void read_knobs() {
   Knobs k;
   struct { const char* name; int* dst; } table[] = {
-      {"NT", &k.nt}, {"KW", &k.kw}, {"DEPTH", &k.depth}, {"ROT_SPREAD", &k.rot_spread}, {"XCD_SWIZZLE", &k.xcd_swizzle}, {"WIDE_ORDER_MIN_IDLE", &k.wide_order_min_idle},
+      {"NT", &k.nt}, {"KW", &k.kw}, {"DEPTH", &k.depth}, {"ROT_SPREAD", &k.rot_spread}, {"XCD_SWIZZLE", &k.xcd_swizzle}, {"XCD_CGS", &k.xcd_cgs}, {"WIDE_ORDER_MIN_IDLE", &k.wide_order_min_idle},
       {"PASS_NT", &k.pass_nt}, {"WIDE", &k.wide}, {"WIDE_DEPTH", &k.wide_depth}, {"WIDE_MIN_UNITS", &k.wide_min_units},
       {"WIDE_MIN_BATCH", &k.wide_min_batch}, {"PLAN_WIDE_MIN_UNITS", &k.plan_wide_min_units},
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
       {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
-      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"PLAN_BIG", &k.plan_big}, {"MID_KS64", &k.mid_ks64}, {"LORA_MFMA", &k.lora_mfma}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
+      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"PLAN_BIG", &k.plan_big}, {"LORA_MFMA", &k.lora_mfma}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
       {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
       {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift}, {"SHARE16", &k.share16}, {"SHARE16_MAX_BLOCKS", &k.share16_max_blocks},
   };
@@ -311,6 +311,60 @@ static long wide_grid_units(long rows, int m, int order) {
   }
   return rows * cg_pad;
 }
+// Workgroups of a wide-kernel launch over `rows` tiles in blocks of `xc` column groups x blocks of tiles per XCD
+// (order 4); -1 where 8 XCDs cannot be cut into blocks of that many column groups on this layer.
+static long wide_block_grid_units(long rows, int m, long xc) {
+  const long cgs = (m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
+  if (xc <= 0 || cg_pad % xc != 0 || cg_pad / xc > 8 || 8 % (cg_pad / xc) != 0) return -1;
+  const long tbs = 8 / (cg_pad / xc);
+  return 8 * xc * ((rows + tbs - 1) / tbs);
+}
+// Workgroups of a wide-kernel launch over a plan's list of at most `rows` tiles (or halves of tiles) of `tok` tokens,
+// and the order of its units.  Where the layer's order is the plain one (1: every XCD takes a run of column groups for
+// every tile, so that every XCD's L2 fetches every tile's activations), blocks of column groups x blocks of tiles per
+// XCD (order 4; the blocks of tiles are cut on the device from the list's real length) make the L2s fetch fewer bytes
+// once the batch has tokens enough: while the `window` workgroups that an XCD holds at a time walk K, its L2 fetches the
+// weights of their distinct (delta, column group) pairs and the activations of their distinct tiles; with units numbered
+// column group first and about `tiles_per_delta` adjacent tiles per delta, blocks of c column groups fetch
+// c x ceil(window / c / tiles_per_delta) x (a column group's weights) + window / c x (a tile's activations).
+// Measured (order 1 -> blocks): 16 deltas of 4096 x 4096 with 1024 / 2048 tokens 56.4 -> 54.5, 76.5 -> 74.8 us (blocks of
+// 4 or 8); 32 deltas of 4096 x 11008 with 1024 / 4096 tokens 154-158 -> 146, 290-300 -> 284 us (blocks of 12; of 24:
+// 165 and 296); 64 deltas of 8192 x 28672 with 256 / 1024 tokens: the plain order stays ahead (644 against 662 us in
+// blocks of 14).  The knob xcd_cgs forces a block size (> 0) or the plain order (-1).
+static unsigned plan_wide_grid(Sparse24Args& b, long rows, int m, int tok, int prob_n, int n_deltas, int window) {
+  const long cgs = (m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
+  const long forced = knobs().xcd_cgs;
+  long best = cg_pad / 8;
+  if (b.xcd_swizzle == 1 && forced >= 0) {
+    const double groups = n_deltas < prob_n ? n_deltas : prob_n;
+    const double tpd = prob_n / (tok * groups) > 1.0 ? prob_n / (tok * groups) : 1.0;          // tiles per delta
+    const double per_tile = prob_n / groups < tok ? prob_n / groups : tok;                      // tokens per tile
+    const double w_cg = 512.0 * b.k * 0.375, x_tile = per_tile * b.k * 2.0;
+    auto fetched = [&](long xc) {
+      const double tiles = (double)window / xc > 1.0 ? (double)window / xc : 1.0;
+      double deltas = tiles / tpd > 1.0 ? tiles / tpd : 1.0;
+      if (deltas > groups) deltas = groups;
+      return xc * deltas * w_cg + tiles * x_tile;
+    };
+    double best_bytes = fetched(best);
+    for (long xc = 1; xc <= cg_pad; xc++) {
+      if (cg_pad % xc != 0 || cg_pad / xc > 8 || 8 % (cg_pad / xc) != 0) continue;
+      if (forced > 0) {
+        if (xc == forced) best = xc;
+        continue;
+      }
+      // (tiles of a plan are ragged: a block of tiles is shared by two XCDs at least, so that the XCDs' loads stay alike;
+      // blocks of all 24 column groups of 4096 x 11008 measured 4 % behind the plain order)
+      if (cg_pad / xc >= 2 && fetched(xc) < 0.95 * best_bytes) { best = xc; best_bytes = fetched(xc); }
+    }
+  }
+  if (best != cg_pad / 8 || (forced > 0 && best == forced && b.xcd_swizzle == 1)) {
+    b.xcd_swizzle = 4;
+    b.xcd_cgs = (int)best;
+    return (unsigned)wide_block_grid_units(rows, m, best);
+  }
+  return (unsigned)wide_grid_units(rows, m, b.xcd_swizzle);
+}
 int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   const long cgs = (a.m / 128 + 3) / 4;
@@ -321,7 +375,45 @@ int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   Sparse24Args b = a;
   if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
   b.xcd_swizzle = wide_unit_order(a.m);
-  const unsigned grid = (unsigned)wide_grid_units((long)a.n_groups * chunks, a.m, b.xcd_swizzle);
+  unsigned grid = (unsigned)wide_grid_units((long)a.n_groups * chunks, a.m, b.xcd_swizzle);
+  // Uniform launches: an XCD takes a block of column groups x a block of token tiles (order 4) where that makes its
+  // L2 fetch fewer bytes than a run of column groups for every tile (order 1).  While the workgroups that an XCD holds at
+  // a time (32 CUs x 1 or 2) walk K, its L2 fetches the packed weights of their distinct column groups and the
+  // activations of their distinct tiles once each: with units numbered column group first, a window of W units over
+  // blocks of c column groups fetches c x (weights of a column group) + W / c x (activations of a tile), least near
+  // c = sqrt(W x tile / column group).  Measured (order 1 -> the rule): 4096 x 4096 with 640 / 1024 / 1536 / 2048 tokens
+  // 28.3 -> 27.1, 32.1 -> 30.6, 43.8 -> 41.6, 50.5 -> 46.8 us; 8192 x 8192 with 1000 tokens 81.2 -> 79.7 us; 11008 x 4096 with
+  // 1280 tokens 92.5 -> 88.6 us; 4096 x 11008 and 8192 x 28672 the same either way (blocks of 14 column groups on the
+  // latter, which a count over the whole launch instead of the window would pick, measured 1.7 % slower).
+  // The sums do not depend on which workgroup takes which unit.
+  const bool eight_waves = !a.tiles && ((tok == 32 && units <= knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits)) ||
+                                        (tok != 32 && units <= knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits)));
+  if (!a.tiles && b.xcd_swizzle == 1 && knobs().xcd_cgs >= 0) {
+    const long rows = (long)a.n_groups * chunks;
+    const double w_cg = 512.0 * a.k * 0.375, x_tile = (double)tok * a.k * 2.0;
+    const long window = 32 * (eight_waves ? 1 : 2);                       // workgroups an XCD holds at a time
+    auto fetched = [&](long xc) {
+      const long tbs = 8 / (cg_pad / xc);
+      long slots = xc * ((rows + tbs - 1) / tbs);
+      if (slots > window) slots = window;
+      return (double)xc * w_cg + (double)((slots + xc - 1) / xc) * x_tile;
+    };
+    long best = cg_pad / 8;
+    double best_bytes = fetched(best);
+    for (long xc = 1; xc <= cg_pad; xc++) {
+      if (cg_pad % xc != 0 || cg_pad / xc > 8 || 8 % (cg_pad / xc) != 0) continue;
+      if (knobs().xcd_cgs > 0) {                                           // (forced, for measurements)
+        if (xc == knobs().xcd_cgs) best = xc;
+        continue;
+      }
+      if (fetched(xc) < 0.95 * best_bytes) { best = xc; best_bytes = fetched(xc); }
+    }
+    if (best != cg_pad / 8 || knobs().xcd_cgs > 0) {
+      b.xcd_swizzle = 4;
+      b.xcd_cgs = (int)best;
+      grid = (unsigned)wide_block_grid_units(rows, a.m, best);
+    }
+  }
   if (tok == 32 && units <= knob_or(knobs().wide32_ksplit_max_units, kWide32KSplitMaxUnits))
     hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, false, 2>), dim3(grid), dim3(512), 0, st, b);
   else if (tok == 32)
@@ -820,6 +912,10 @@ long triteia_hip_wide_grid_units(long rows, int prob_m, int order) {
   if (order == 3 && ((prob_m / 128 + 3) / 4) % 8 == 0) order = 1;
   return wide_grid_units(rows, prob_m, order);
 }
+long triteia_hip_wide_block_grid_units(long rows, int prob_m, int block_column_groups) {
+  if (rows <= 0 || prob_m < 128) return 0;
+  return wide_block_grid_units(rows, prob_m, block_column_groups);
+}
 int triteia_hip_planned_tile_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   if (prob_n <= 0 || n_deltas <= 0 || prob_m <= 0 || prob_k <= 0) return 0;
   if (mid_big(prob_n, n_deltas, prob_m, prob_k)) return 64;
@@ -906,19 +1002,6 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     const int forced = knobs().pass_nt;
     if ((forced == 1 || forced == 2 || forced == 4) && 16 * forced <= tile) pass_nt = forced;
   }
-  // A plan that also lists its tokens in 64-token tiles, on a layer where even the host's bound on those tiles makes at
-  // most one workgroup per CU: the 64-token build on eight wavefronts (K halved inside the workgroup) takes that list.
-  if (knobs().mid_ks64 && plan_has_big(prob_n, n_deltas) && prob_k % 128 == 0 && (long)prob_n * prob_k * 2 < (1L << 32) &&
-      (long)L.max_big * (((prob_m / 128 + 3) / 4 + 7) / 8 * 8) <= knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits)) {
-    a.xcd_swizzle = wide_unit_order(prob_m);
-    a.tiles = reinterpret_cast<const int4*>(ws + L.big);
-    a.tiles_alt = nullptr;
-    a.n_groups_dev = ws + L.header + 6;
-    a.n_groups = L.max_big;
-    hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true, 2>), dim3((unsigned)wide_grid_units(a.n_groups, prob_m, a.xcd_swizzle)), dim3(512), 0,
-                       static_cast<hipStream_t>(stream), a);
-    return check_launch("sparse24_wide_kernel (plan's 64-token tiles, eight wavefronts)");
-  }
   if (mid) a.xcd_swizzle = wide_unit_order(prob_m);
   if (mid && mid_big(prob_n, n_deltas, prob_m, prob_k)) {
     // the plan's own list of 64-token tiles, whole, on the 64-token build
@@ -928,7 +1011,7 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     a.n_groups_dev = ws + L.header + 6;
     a.n_groups = L.max_big;
     if ((long)a.n_groups * cg_pad > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units");
-    hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3((unsigned)wide_grid_units(a.n_groups, prob_m, a.xcd_swizzle)), dim3(256), 0,
+    hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3(plan_wide_grid(a, a.n_groups, prob_m, 64, prob_n, n_deltas, 64)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), a);
     if (int e = check_launch("sparse24_wide_kernel (plan tiles)")) return e;
   } else if (mid) {
@@ -937,14 +1020,14 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     const long units32 = (long)a.n_groups * (tile == 64 ? 2 : 1) * cg_pad;   // in 32-token tiles, on the plan's bound
     if (mid_deep(prob_n, n_deltas, prob_m, tile) && units32 <= 0x7fffffffL) {
       a.tile_halves = tile == 64;
-      hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, true>), dim3((unsigned)wide_grid_units((long)a.n_groups * (tile == 64 ? 2 : 1), prob_m, a.xcd_swizzle)), dim3(256), 0,
+      hipLaunchKernelGGL((sparse24_wide_kernel<2, 32, true>), dim3(plan_wide_grid(a, (long)a.n_groups * (tile == 64 ? 2 : 1), prob_m, 32, prob_n, n_deltas, 64)), dim3(256), 0,
                          static_cast<hipStream_t>(stream), a);
       a.tile_halves = 0;
     } else if (tile == 32)
-      hipLaunchKernelGGL((sparse24_wide_kernel<1, 32, true>), dim3((unsigned)wide_grid_units(a.n_groups, prob_m, a.xcd_swizzle)), dim3(256), 0,
+      hipLaunchKernelGGL((sparse24_wide_kernel<1, 32, true>), dim3(plan_wide_grid(a, a.n_groups, prob_m, 32, prob_n, n_deltas, 64)), dim3(256), 0,
                          static_cast<hipStream_t>(stream), a);
     else
-      hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3((unsigned)wide_grid_units(a.n_groups, prob_m, a.xcd_swizzle)), dim3(256), 0,
+      hipLaunchKernelGGL((sparse24_wide_kernel<1, 64, true>), dim3(plan_wide_grid(a, a.n_groups, prob_m, 64, prob_n, n_deltas, 64)), dim3(256), 0,
                          static_cast<hipStream_t>(stream), a);
     if (int e = check_launch("sparse24_wide_kernel (plan tiles)")) return e;
   } else

@@ -41,6 +41,7 @@ SIGNATURES = {
     "triteia_hip_planned_tile_kernel": (_c_int, [_c_int, _c_int, _c_int, _c_int]),
     "triteia_hip_wide_unit_order": (_c_int, [_c_int]),
     "triteia_hip_wide_grid_units": (ctypes.c_long, [ctypes.c_long, _c_int, _c_int]),
+    "triteia_hip_wide_block_grid_units": (ctypes.c_long, [ctypes.c_long, _c_int, _c_int]),
     "triteia_hip_route_plan": (_c_int, [_c_vp, _c_int, _c_int, _c_int, _c_vp, _c_sz, _c_int, _c_vp]),
     "triteia_hip_bgmv": (_c_int, [_c_vp] * 4 + [_c_int] * 5 + [_c_float, _c_int, _c_vp]),
     "triteia_hip_sgmv": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp]),
