@@ -62,7 +62,11 @@ TRITEIA_HIP_API void triteia_hip_reload_env(void);
  * reference as mul_2_4 (triteia/csrc/ops/ops.cpp:88-116).
  * workspace: the reference's lock array (>= prob_m/128*max_par int32 zeros); it
  * is accepted, never read or written, and therefore left all-zero.
- * groupsize must be -1 (per-channel scales).  thread_k, thread_m, sms, max_par
+ * groupsize, in the reference's unit of compressed k (marlin_nm.cu:68): -1 = one scale per output column, s [1, m];
+ * 64 = one per column and 128 dense k, s [prob_k / 128, m] with every run of 8 columns stored in the order
+ * 0 4 1 5 2 6 3 7 (triteia/python/ops/utils/sparsity.py:54-57), prob_k % 128 == 0; anything else ERR_KERN_SHAPE
+ * (the reference instantiates the same two, marlin_nm.cu:102-111).  The batched and routed entry points below take
+ * -1 only.  thread_k, thread_m, sms, max_par
  * are the reference's tuning knobs; they are accepted and ignored.
  * Shape rules: prob_m % 128 == 0 and prob_k % 64 == 0, else ERR_PROB_SHAPE. */
 TRITEIA_HIP_API int triteia_hip_mul_2_4(const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m, int prob_n,

@@ -14,6 +14,11 @@ checkout):
   encode_2_4_nonzero ............ triteia/python/ops/utils/sparsity.py:167-290
   mask_2_4 ...................... triteia/python/ops/utils/sparsity.py:99-118
   pack_reference ................ triteia/python/nn/linear.py:79-141
+  scale_perm_2_4, store/load_group_scales, pack_reference_grouped
+                                  triteia/python/ops/utils/sparsity.py:54-57,
+                                  triteia/python/nn/linear.py:104-118 (scales per
+                                  column and group of 128 dense k), used by the
+                                  kernel as marlin.cuh:199-209,342-346,378-380
   pack_explicit ................. same layout, positions given explicitly
   unpack ........................ inverse of the two packers (the dense weight
                                   the reference's tests multiply by,
@@ -34,6 +39,14 @@ How each is pinned (see tests/test_oracle_*.py):
   pack_*/unpack: exact integer round trips, brute force at the minimum legal
       size, single-nonzero closed forms.
   GEMM / routing / LoRA: float64 textbook loops on tiny inputs.
+  grouped scales: the stored order against the golden table of the reference's
+      own `_get_perms_2_4`; the arithmetic against a plain loop and against the
+      per-column form when all groups carry the same scales.  No test, caller or
+      fixture of the reference exercises grouped scales on this path (its module
+      asserts groupsize == -1, linear.py:27), so which column a stored scale
+      multiplies inside the reference's kernel is taken from reading
+      marlin.cuh:199-209,378-380 together with the weight permutation: PARITY
+      UNPINNED beyond that.
   mask_2_4 tie-breaking (equal magnitudes inside a group): PARITY UNPINNED --
       the reference uses an unstable argsort there; BASELINE workloads give the
       kept positions explicitly and never depend on it.
@@ -68,6 +81,30 @@ def perm_2_4() -> np.ndarray:
             perm.extend(p + j for p in perm1)
     perm = np.array(perm, dtype=np.int64)
     return perm.reshape(-1, 8)[:, _INTERLEAVE].ravel()
+
+
+def scale_perm_2_4() -> np.ndarray:
+    """Order in which a run of 64 grouped scales is stored (`scale_perm` of `_get_perms_2_4`, sparsity.py:54-57):
+    stored[p] = scale[perm[p]], i.e. inside every run of 8 columns the order 0 4 1 5 2 6 3 7."""
+    return np.array([i * 8 + j for i in range(8) for j in (0, 4, 1, 5, 2, 6, 3, 7)], dtype=np.int64)
+
+
+GROUP_K = 128   # dense k per scale group: groupsize 64 in the launcher's unit of compressed k (marlin_nm.cu:68)
+
+
+def store_group_scales(scales: np.ndarray) -> np.ndarray:
+    """[k/128, m] scales by (group, column) -> the stored tensor of the same shape (linear.py:117,124)."""
+    g, m = scales.shape
+    assert m % 64 == 0
+    return np.ascontiguousarray(scales.reshape(-1, 64)[:, scale_perm_2_4()].reshape(g, m))
+
+
+def load_group_scales(stored: np.ndarray) -> np.ndarray:
+    """Inverse of `store_group_scales`."""
+    g, m = stored.shape
+    out = np.empty((g * m // 64, 64), dtype=stored.dtype)
+    out[:, scale_perm_2_4()] = stored.reshape(-1, 64)
+    return out.reshape(g, m)
 
 
 def perm_2_4_closed_form() -> np.ndarray:
@@ -226,6 +263,23 @@ def pack_reference(weight: np.ndarray, scales: np.ndarray, mask: np.ndarray | No
     return q, reorder_meta(meta16).view(np.int16), scales.reshape(1, m).astype(np.float16)
 
 
+def pack_reference_grouped(weight: np.ndarray, scales: np.ndarray, mask: np.ndarray | None = None):
+    """`pack(weight, scales, trans=True)` of a module with groups of 128 dense k (linear.py:104-124): every
+    weight is divided by the scale of its (group, column); `scales` [k/128, m] by (group, column).  Returns
+    (qweight, meta, stored scales [k/128, m])."""
+    k, m = weight.shape
+    assert k % GROUP_K == 0 and scales.shape == (k // GROUP_K, m)
+    per_row = np.repeat(scales.astype(np.float16), GROUP_K, axis=0)                     # [k, m]
+    if mask is None:
+        mask = mask_2_4(np.ascontiguousarray(weight.T))
+    w = np.rint((weight / per_row).astype(np.float16).astype(np.float32)).astype(np.int32)
+    w = np.clip(w + 8, 0, 15)
+    w = (mask * w.T).astype(np.int32)
+    sparse, meta16 = encode_2_4_nonzero(np.ascontiguousarray(w))
+    q = _pack_nibbles(np.ascontiguousarray(sparse.T))
+    return q, reorder_meta(meta16).view(np.int16), store_group_scales(scales.astype(np.float16))
+
+
 def pack_explicit(q_kept: np.ndarray, lo: np.ndarray, hi: np.ndarray, scales: np.ndarray):
     """Packer with explicit positions (no `!= 0` inference).
 
@@ -293,8 +347,13 @@ def unpack(qweight: np.ndarray, meta: np.ndarray, scales: np.ndarray) -> np.ndar
     reference weight.
     """
     q = unpack_int(qweight, meta)
-    s = np.asarray(scales, dtype=np.float16).reshape(1, -1)
-    return (q.astype(np.float16) * s).astype(np.float16)
+    s = np.asarray(scales, dtype=np.float16)
+    if s.ndim == 2 and s.shape[0] > 1:
+        # grouped: the stored scale of (group of 128 dense k, column) multiplies the dequantised weight in fp16, as
+        # the reference's kernel does ahead of its MMA (marlin.cuh:378-380)
+        assert s.shape[0] * GROUP_K == q.shape[0]
+        return (q.astype(np.float16) * np.repeat(load_group_scales(s), GROUP_K, axis=0)).astype(np.float16)
+    return (q.astype(np.float16) * s.reshape(1, -1)).astype(np.float16)
 
 
 # --------------------------------------------------------------------------

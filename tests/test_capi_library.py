@@ -35,7 +35,7 @@ def test_version_and_error_text():
 @pytest.mark.parametrize("m,n,k,gs,code", [
     (100, 16, 4096, -1, _ffi.ERR_PROB_SHAPE),      # m not a multiple of 128
     (4096, 16, 100, -1, _ffi.ERR_PROB_SHAPE),      # k not a multiple of 64
-    (4096, 16, 4096, 64, _ffi.ERR_KERN_SHAPE),     # grouped scales are not implemented
+    (4096, 16, 4096, 32, _ffi.ERR_KERN_SHAPE),     # scale groups other than 128 dense k (groupsize 64) have no kernel
     (4096, 0, 4096, -1, 0),                        # empty problem is a no-op
 ])
 def test_shape_errors_do_not_need_a_gpu(m, n, k, gs, code):
@@ -47,6 +47,19 @@ def test_shape_errors_do_not_need_a_gpu(m, n, k, gs, code):
         assert _ffi.last_error() != ""
     rc = lib.triteia_hip_bmm_2_4(null, null, null, null, null, m, n, k, null, gs, 0, null, -1, -1, -1, 16)
     assert rc == code
+
+
+def test_grouped_scales_are_for_the_single_matrix_product():
+    """groupsize 64 (scales per column and 128 dense k, marlin_nm.cu:68,102-111) is taken by mul_2_4; the batched and
+    routed launchers, whose group iteration the reference itself has commented out (triteia_nm_bmm.cu:69-71,
+    triteia_nm_sbmm.cu:70-72), answer ERR_KERN_SHAPE; K must be whole groups."""
+    lib = _ffi.lib()
+    null = ctypes.c_void_p(0)
+    assert lib.triteia_hip_mul_2_4(null, null, null, null, null, 4096, 0, 4096, null, 64, 0, null, -1, -1, -1, 16) == 0
+    assert lib.triteia_hip_mul_2_4(null, null, null, null, null, 4096, 16, 4096, null, 64, 0, null, -1, -1, -1, 16) == _ffi.ERR_ARGUMENT
+    assert lib.triteia_hip_mul_2_4(null, null, null, null, null, 4096, 16, 4160, null, 64, 0, null, -1, -1, -1, 16) == _ffi.ERR_PROB_SHAPE
+    assert lib.triteia_hip_bmm_2_4(null, null, null, null, null, 4096, 16, 4096, null, 64, 0, null, -1, -1, -1, 16) == _ffi.ERR_KERN_SHAPE
+    assert lib.triteia_hip_sbmm_2_4(*([null] * 8), 4096, 16, 4096, 1, null, 64, 0, null, -1, -1, -1, 16) == _ffi.ERR_KERN_SHAPE
 
 
 def test_other_argument_errors():

@@ -129,3 +129,17 @@ def test_tp_shards_are_packed_independently():
     qs, ss, ms = gen.torch_weight_to_sparse_marlin(w24, s, tp_size=2, chunk_by="row", device="cpu")
     parts = [orc.unpack(q.numpy(), me.numpy(), sc.numpy()) for q, sc, me in zip(qs, ss, ms)]
     assert np.array_equal(np.concatenate(parts, axis=0), full)
+
+
+def test_group_scales_codec_matches_the_oracle():
+    from triteia_amd.python.ops.utils.sparsity import pack_group_scales, unpack_2_4, unpack_group_scales
+    rng = np.random.default_rng(5)
+    k, m = 256, 128
+    s = (np.abs(rng.standard_normal((k // 128, m))) * 0.01 + 0.005).astype(np.float16)
+    stored = pack_group_scales(torch.from_numpy(s))
+    assert np.array_equal(stored.numpy(), orc.store_group_scales(s))
+    assert np.array_equal(unpack_group_scales(stored).numpy(), s)
+    w = (rng.standard_normal((k, m)) * 0.05).astype(np.float16)
+    qw, meta, st = orc.pack_reference_grouped(w, s)
+    W = unpack_2_4(torch.from_numpy(qw), torch.from_numpy(meta), torch.from_numpy(st))
+    assert np.array_equal(W.numpy(), orc.unpack(qw, meta, st))

@@ -70,6 +70,42 @@ def test_matmul_4bit_2_4(ops, n, k, m, seed):
     check_close(out, ref, what="matmul_4bit_2_4")
 
 
+@pytest.mark.parametrize("n,k,m,seed", [
+    (1, 256, 256, 31), (16, 256, 128, 32), (17, 512, 256, 33), (33, 512, 384, 34), (100, 1024, 640, 35),
+    (300, 384, 256, 36),
+    (16, 4096, 4096, 37),                             # BASELINE config 0's shape with a scale per 128 k and column
+])
+def test_matmul_with_scales_per_group_of_k(ops, n, k, m, seed):
+    """groupsize 64 of the reference's launcher (marlin_nm.cu:68,102-111): `s` is [k/128, m] in the stored order.
+    Against the oracle, which scales the dequantised weight in fp16 as the reference's kernel does; and, with all
+    groups alike, against the per-column product of the same weights."""
+    say(f"matmul grouped scales n={n} k={k} m={m} seed={seed}")
+    rng = np.random.default_rng(seed)
+    qw, meta, _ = make_deltas(1, k, m, seed)
+    s_true = rng.uniform(0.005, 0.02, size=(k // 128, m)).astype(np.float16)
+    stored = orc.store_group_scales(s_true)
+    x = activations(n, k, seed + 1)
+    ref = orc.matmul_4bit_2_4(qw[0], x, meta[0], stored)
+    gq, gm, gs, gx = to_gpu(qw[0], meta[0], stored, x)
+    out = ops.matmul_4bit_2_4(gq, gx, gm, gs)
+    torch.cuda.synchronize()
+    assert out.shape == (n, m) and out.dtype == torch.float16
+    check_close(out, ref, what="matmul_4bit_2_4 (grouped scales)")
+    # every group with the scales of group 0: the per-column product
+    flat = orc.store_group_scales(np.repeat(s_true[:1], k // 128, axis=0))
+    one = ops.matmul_4bit_2_4(gq, gx, gm, torch.from_numpy(flat).to(DEV))
+    per_column = ops.matmul_4bit_2_4(gq, gx, gm, torch.from_numpy(s_true[:1]).to(DEV))
+    torch.cuda.synchronize()
+    check_close(one, per_column.float().cpu().numpy().astype(np.float64), tol=1e-3, what="grouped == per-column")
+
+
+def test_scale_groups_other_than_128_k_are_refused(ops):
+    qw, meta, _ = make_deltas(1, 256, 128, 40)
+    gq, gm, gx = to_gpu(qw[0], meta[0], activations(4, 256, 41))
+    with pytest.raises(RuntimeError, match="groupsize=32"):
+        ops.matmul_4bit_2_4(gq, gx, gm, torch.ones((4, 128), dtype=torch.float16, device=DEV))
+
+
 @pytest.mark.parametrize("kernel", ["wide64", "wide64ks", "tile256", "wide32", "wide32ks"])
 @pytest.mark.parametrize("n,k,m,seed", [
     (64, 128, 512, 21), (128, 128, 512, 22), (128, 256, 128, 23),      # one tile, 1 and 2 k steps

@@ -26,6 +26,52 @@ def test_scale_perm_single_is_identity():
     assert np.array_equal(G["scale_perm_single_2_4"], np.arange(64))
 
 
+def test_group_scale_order_matches_reference_table():
+    # scales per group of K are stored with every run of 8 columns in the order 0 4 1 5 2 6 3 7 (sparsity.py:54-57)
+    assert np.array_equal(orc.scale_perm_2_4(), G["scale_perm_2_4"])
+    assert np.array_equal(np.sort(orc.scale_perm_2_4()), np.arange(64))
+    s = np.arange(3 * 128, dtype=np.float16).reshape(3, 128)
+    stored = orc.store_group_scales(s)
+    # column c of a run of 8 sits at position 0 2 4 6 1 3 5 7 [c] of that run
+    for g in range(3):
+        for col in range(128):
+            assert stored[g, col // 8 * 8 + (0, 2, 4, 6, 1, 3, 5, 7)[col % 8]] == s[g, col]
+    assert np.array_equal(orc.load_group_scales(stored), s)
+
+
+def test_grouped_scales_against_a_plain_loop_and_the_per_column_form():
+    rng = np.random.default_rng(77)
+    k, m, T = 256, 256, 3
+    w = (rng.standard_normal((k, m)) * 0.05).astype(np.float16)
+    mask = orc.mask_2_4(np.ascontiguousarray(np.abs(w.T.astype(np.float32)) + rng.random((m, k)).astype(np.float32) * 1e-3))
+    # (scales large enough that no kept weight reaches -8: the reference's packer takes nibble 0 for a pruned entry)
+    s = (np.abs(rng.standard_normal((k // 128, m))) * 0.01 + 0.035).astype(np.float16)
+    qw, meta, stored = orc.pack_reference_grouped(w, s, mask)
+    assert stored.shape == (k // 128, m) and stored.dtype == np.float16
+    W = orc.unpack(qw, meta, stored)
+    q = orc.unpack_int(qw, meta)
+    # every weight: its integer times the scale of (its group of 128 rows, its column), rounded to fp16; the integer is
+    # the weight divided by that scale, rounded, clamped to int4, zero where pruned
+    for kk in range(0, k, 5):
+        for c in range(0, m, 3):
+            sc = s[kk // 128, c]
+            assert W[kk, c] == np.float16(np.float16(q[kk, c]) * sc)
+            want = int(np.clip(np.rint(np.float32(np.float16(w[kk, c] / sc))), -8, 7)) if mask[c, kk] else 0
+            assert q[kk, c] == want, (kk, c)
+    x = rng.standard_normal((T, k)).astype(np.float16)
+    y = orc.matmul_4bit_2_4(qw, x, meta, stored)
+    for t in range(T):
+        for c in range(0, m, 7):
+            acc = sum(float(x[t, kk]) * float(W[kk, c]) for kk in range(k))
+            assert abs(acc - y[t, c]) < 1e-9
+    # all groups alike: the per-column result
+    s1 = s[:1]
+    qw1, meta1, stored1 = orc.pack_reference_grouped(w, np.repeat(s1, k // 128, axis=0), mask)
+    qwc, metac, sc1 = orc.pack_reference(w, s1, mask)
+    assert np.array_equal(qw1, qwc) and np.array_equal(meta1, metac)
+    assert np.array_equal(orc.matmul_4bit_2_4(qw1, x, meta1, stored1), orc.matmul_4bit_2_4(qwc, x, metac, sc1))
+
+
 @pytest.mark.parametrize("m,ncols", [(64, 2), (128, 8), (256, 8), (256, 16), (512, 4)])
 def test_meta_offsets_match_reference_table(m, ncols):
     off = orc.meta_scatter_offsets(m, ncols)

@@ -56,7 +56,8 @@ struct Sparse24Args {
   long qweight_stride;      // vectors between deltas
   const uint4_t* meta;      // [N][k/32][m/4] 16-byte vectors (physical order)
   long meta_stride;         // vectors between deltas
-  const _Float16* scales;   // [N][m]
+  const _Float16* scales;   // [N][m]; with scale_groups > 0 (GS builds): [N][scale_groups][m], one row per 128 dense k,
+                            // each run of 8 columns stored in the order 0 4 1 5 2 6 3 7 (the reference's grouped layout)
   long scales_stride;       // elements between deltas
   _Float16* out;            // [T, m]
   long out_stride;          // elements between rows
@@ -114,6 +115,7 @@ struct Sparse24Args {
   // 1: the plan's tiles hold up to 64 tokens and the 32-token build of the wide kernel takes each as two halves
   // (workgroups 2g and 2g + 1 of a column group; a half without tokens returns at once)
   int tile_halves;
+  int scale_groups;         // 0: one scale per output column; else k / 128 groups of K, each with a scale per column
 };
 
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
@@ -165,6 +167,7 @@ struct StepFrag {
   uint4_t mt[2];        // metadata vectors (b1 = 0, 1)
   uint4_t xa[NT][2];    // B slots 0..7 for u = 0, 1
   uint4_t xb[NT][2];    // B slots 8..15 for u = 0, 1
+  uint4_t gs[4];        // grouped scales only: the step's scales of this lane's 4 x 8 output columns
 };
 
 // weights and metadata of one step, requested ahead of a tile pass
@@ -203,7 +206,9 @@ struct TileCtx {
 // One pass over K for up to 16*NTT tokens of one group: loads, sparse MFMAs, cross-wave
 // reduction, scaled fp16 store.  `first` = index of the pass's first token in the group's list.
 // NPRE: the weights of this wave's first NPRE (<= DEPTH) steps are already on their way in `pre`.
-template <int NTT, int KW, int DEPTH, int NPRE = 0>
+// GS: grouped scales (one scale per column and 128-k step instead of one per column): each step's MFMAs start from
+// zero and their sums enter the running sums times the step's scales.
+template <int NTT, int KW, int DEPTH, int NPRE = 0, bool GS = false>
 __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int first, int cnt,
                                           float (*red)[16][kRedStride], int* s_rows, const WPre* pre = nullptr) {
   const int r = c.r, q = c.q, wave = c.wave;
@@ -228,6 +233,12 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
     for (int a = 0; a < 4; a++) f.wq[a] = wp[a];
     f.mt[0] = mp[0];
     f.mt[1] = mp[8];
+    if constexpr (GS) {
+      // D rows 4q + j of this lane = columns 8 (4q + j) .. + 7 of the column block
+      const _Float16* sp = c.sc + (long)phys(st) * p.m + 32 * q;
+#pragma unroll
+      for (int j = 0; j < 4; j++) f.gs[j] = *reinterpret_cast<const uint4_t*>(sp + 8 * j);
+    }
   };
 
   // Start-up order matters (vector loads return in order): first the tiny per-lane read of
@@ -264,7 +275,8 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
   // The scales of this thread's 8 output features, for the epilogue: requested here, behind the first
   // weights, so that no wait for them can land ahead of a request (requested before the loop over
   // passes they were waited for at the loop's entry: a full memory round trip before the first weights).
-  const half8_t sv = *reinterpret_cast<const half8_t*>(c.sc + c.col0 + (c.tid & ((1 << c.nblk_shift) - 1)) * 8);
+  half8_t sv = {1, 1, 1, 1, 1, 1, 1, 1};
+  if constexpr (!GS) sv = *reinterpret_cast<const half8_t*>(c.sc + c.col0 + (c.tid & ((1 << c.nblk_shift) - 1)) * 8);
 
   // Every lane always loads from a valid address, so that the number of loads per step is
   // fixed and the hardware load counter can be waited on exactly (the output columns of the
@@ -306,6 +318,56 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
     const bool tail = tr0 + 4 > k_rows;            // wave-uniform: only the last, partial step
     const bool ok_a = (tr0 + (q >> 1)) < k_rows;
     const bool ok_b = (tr0 + 2 + (q >> 1)) < k_rows;
+    if constexpr (GS) {
+      // (K is a whole number of steps here.)  Column by column: the two MFMAs of a column (k halves u = 0, 1) start
+      // from zero, and their sum enters the running sum times the scale of (this step, that column).
+      half16_t b[2][NTT];
+#pragma unroll
+      for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int nt = 0; nt < NTT; nt++) {
+          typedef uint32_t uint8_t_v __attribute__((ext_vector_type(8)));
+          const uint8_t_v bb = {f.xa[nt][u][0], f.xa[nt][u][1], f.xa[nt][u][2], f.xa[nt][u][3],
+                                f.xb[nt][u][0], f.xb[nt][u][1], f.xb[nt][u][2], f.xb[nt][u][3]};
+          b[u][nt] = __builtin_bit_cast(half16_t, bb);
+        }
+#pragma unroll
+      for (int cc = 0; cc < 8; cc++) {
+        const int w = cc & 3, b2 = cc >> 2;
+        float4_t part[NTT];
+#pragma unroll
+        for (int nt = 0; nt < NTT; nt++) part[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+          uint4_t av;
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            uint32_t word = f.wq[a][w];
+            if (b2) word >>= 8;
+            av[a] = u ? dequant_odd(word) : dequant_even(word);
+          }
+          const half8_t A = __builtin_bit_cast(half8_t, av);
+          const int idx = (int)f.mt[(cc >> 1) & 1][(cc & 1) * 2 + u];
+#pragma unroll
+          for (int nt = 0; nt < NTT; nt++) {
+            if (b2)
+              part[nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A, b[u][nt], part[nt], idx, 0, 1);
+            else
+              part[nt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A, b[u][nt], part[nt], idx, 0, 0);
+          }
+        }
+        // column cc of a run of 8 is stored at position 0 2 4 6 1 3 5 7 [cc] of the run
+        constexpr int kPos[8] = {0, 2, 4, 6, 1, 3, 5, 7};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const half2_t pair = bits_h2(f.gs[j][kPos[cc] >> 1]);
+          const float sc = (float)pair[kPos[cc] & 1];
+#pragma unroll
+          for (int nt = 0; nt < NTT; nt++) acc[cc][nt][j] = __builtin_fmaf(part[nt][j], sc, acc[cc][nt][j]);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < 2; u++) {
       half16_t b[NTT];
@@ -418,8 +480,8 @@ __device__ __forceinline__ void tile_pass(const Sparse24Args& p, TileCtx& c, int
 // take the cheaper code path (fewer activation loads and MFMAs) at the same register budget.
 // EAGER: fused routing with group g = delta g (Sparse24Args::raw_static): the weights of the first
 // step are requested at once, together with the indices, instead of one memory round trip later.
-template <int NT, int KW, int DEPTH, bool EAGER = false>
-__global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2 ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
+template <int NT, int KW, int DEPTH, bool EAGER = false, bool GS = false>
+__global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 && !GS ? 3 : 2) : (NT == 2 && !GS ? 2 : 1))) void sparse24_grouped_kernel(const Sparse24Args p) {
   // steps per wave requested ahead of the routing in the EAGER build (the 32- and 64-token builds
   // also hold narrower passes with a ring of their own depth: one step fits them all)
   constexpr int NPRE = EAGER ? (NT == 1 ? DEPTH : 1) : 0;
@@ -468,7 +530,7 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   auto bind_delta = [&](int delta) {
     c.qw_lane = p.qweight + (long)delta * p.qweight_stride + (long)cb * 64 + 4 * c.ra;
     c.mt_lane = p.meta + (long)delta * p.meta_stride + (long)(cb * 2 + (c.ra >> 3)) * 16 + (c.ra & 7);
-    c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;
+    c.sc = p.scales + (long)delta * p.scales_stride + cb * 128;   // (GS: row 0 of the delta's groups)
     // side-by-side deltas start their walks spread around the ring of steps (by the delta's index,
     // so that a result does not depend on where the weights happen to lie in memory)
     // (32-bit arithmetic: a 64-bit remainder is a routine of some 150 instructions ahead of the first request;
@@ -610,11 +672,11 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 ? 3 : 2) : (NT == 2
   for (; t0 < count; t0 += gridDim.y * 16 * NT) {
     const int cnt = min(count - t0, 16 * NT);
     if (NT == 1 || cnt <= 16) {
-      tile_pass<1, KW, (NT == 1 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);
+      tile_pass<1, KW, (NT == 1 ? DEPTH : 2), 0, GS>(p, c, start + t0, cnt, red, s_rows);
     } else if (NT == 2 || cnt <= 32) {
-      tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2)>(p, c, start + t0, cnt, red, s_rows);
+      tile_pass<(NT >= 2 ? 2 : 1), KW, (NT == 2 ? DEPTH : 2), 0, GS>(p, c, start + t0, cnt, red, s_rows);
     } else {
-      tile_pass<NT, KW, DEPTH>(p, c, start + t0, cnt, red, s_rows);
+      tile_pass<NT, KW, DEPTH, 0, GS>(p, c, start + t0, cnt, red, s_rows);
     }
     // the next pass over this group's tokens reuses s_rows / red
     if (t0 + gridDim.y * 16 * NT < count) lds_barrier();

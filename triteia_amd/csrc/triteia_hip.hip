@@ -96,9 +96,15 @@ const Knobs& knobs() {
 // value of a knob whose default depends on the launch
 inline int knob_or(int v, long dflt) { return v == kUnset ? (int)dflt : v; }
 
-int check_gemm_shape(int prob_m, int prob_n, int prob_k, int groupsize) {
-  if (groupsize != -1)
-    return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "groupsize=%d: only per-channel scales (groupsize=-1) are implemented", groupsize);
+// Scale groups along K that the launchers accept, in the reference's unit (compressed k, i.e. dense k / 2): -1, one scale
+// per column, and 64 = 128 dense k = one K step of the kernels (marlin_nm.cu:68,102-111: group_blocks -1 or 4).
+constexpr int kGroupsize = 64;
+int check_gemm_shape(int prob_m, int prob_n, int prob_k, int groupsize, bool grouped_ok = false) {
+  if (groupsize != -1 && !(grouped_ok && groupsize == kGroupsize))
+    return fail(TRITEIA_HIP_ERR_KERN_SHAPE, grouped_ok ? "groupsize=%d: scales per column (groupsize=-1) or per column and 128 dense k (groupsize=64) are implemented"
+                                                       : "groupsize=%d: only per-channel scales (groupsize=-1) are implemented by this entry point", groupsize);
+  if (groupsize != -1 && prob_k % 128 != 0)
+    return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "k=%d is not a whole number of scale groups of 128", prob_k);
   if (prob_m < 0 || prob_n < 0 || prob_k < 0 || prob_m % 128 != 0 || prob_k % 64 != 0)
     return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "problem (m=%d, n=%d, k=%d) needs m %% 128 == 0 and k %% 64 == 0", prob_m, prob_n, prob_k);
   return TRITEIA_HIP_OK;
@@ -251,6 +257,24 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
 #undef TRY
 #undef TRY_EAGER
   return fail(TRITEIA_HIP_ERR_KERN_SHAPE, "no kernel variant for NT=%d KW=%d DEPTH=%d", nt, kw, depth);
+}
+
+// One matrix whose scales come per column and 128-k step (Sparse24Args::scale_groups): the streaming kernel's GS build,
+// whole column blocks, four wavefronts, one step in flight, the tokens in passes of 16 or 32 spread over blockIdx.y
+// (a compatibility path: the reference's own module and converter never produce such scales).
+int launch_grouped_scales(Sparse24Args a, int tokens, hipStream_t st) {
+  a.n_groups = 1;
+  a.uniform_count = tokens;
+  a.uniform_stride = tokens;
+  a.delta_step = 0;
+  const int nt = tokens <= 16 ? 1 : 2;
+  long tsplit = (tokens + 16 * nt - 1) / (16 * nt);
+  if (tsplit > 65535) tsplit = 65535;
+  const long cb_pad = ((long)(a.m / 128) + 7) / 8 * 8;
+  const dim3 grid((unsigned)cb_pad, (unsigned)tsplit, 1);
+  if (nt == 1) hipLaunchKernelGGL((sparse24_grouped_kernel<1, 4, 1, false, true>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((sparse24_grouped_kernel<2, 4, 1, false, true>), grid, dim3(256), 0, st, a);
+  return check_launch("sparse24_grouped_kernel (grouped scales)");
 }
 
 void fill_weights(Sparse24Args& a, const void* A, const void* B, const void* meta, void* C, const void* s, int prob_m,
@@ -670,13 +694,18 @@ int triteia_hip_mul_2_4(const void* A, const void* B, const void* meta, void* C,
                         int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k, int thread_m,
                         int sms, int max_par) {
   (void)workspace; (void)thread_k; (void)thread_m; (void)sms; (void)max_par;
-  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, groupsize)) return e;
+  if (int e = check_gemm_shape(prob_m, prob_n, prob_k, groupsize, true)) return e;
   if (prob_m == 0 || prob_n == 0 || prob_k == 0) return TRITEIA_HIP_OK;
   if (!A || !B || !meta || !C || !s) return fail(TRITEIA_HIP_ERR_ARGUMENT, "mul_2_4: null tensor pointer");
   DeviceGuard g(dev);
   if (!g.ok) return fail(TRITEIA_HIP_ERR_RUNTIME, "cannot select device %d", dev);
   Sparse24Args a;
   fill_weights(a, A, B, meta, C, s, prob_m, prob_k, 1);
+  if (groupsize != -1) {
+    a.scale_groups = prob_k / 128;
+    a.scales_stride = (long)a.scale_groups * prob_m;
+    return launch_grouped_scales(a, prob_n, static_cast<hipStream_t>(stream));
+  }
   return launch_uniform(a, prob_n, prob_n, 0, 1, static_cast<hipStream_t>(stream));
 }
 

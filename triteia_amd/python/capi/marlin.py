@@ -40,7 +40,8 @@ def _check_packed(B, meta, s, prob_m, prob_k, lead=()):
 
 def mul_2_4(A, B, meta, C, s, workspace, thread_k=-1, thread_m=-1, sms=-1, max_par=16):
     """C = A @ W for one packed weight.  A [n, k] fp16, B [k/32, 2m] int32,
-    meta [m, k/16] int16, C [n, m] fp16, s [1, m] fp16, workspace >= m/128*max_par zeros
+    meta [m, k/16] int16, C [n, m] fp16, s [1, m] fp16 (or [k/128, m]: scales per group of 128
+    dense k in the reference's stored order, `sparsity.pack_group_scales`), workspace >= m/128*max_par zeros
     (kept for signature parity; never touched)."""
     _gemm_checks(A, B, meta, C, s)
     if A.dim() != 2 or C.dim() != 2:
@@ -54,7 +55,7 @@ def mul_2_4(A, B, meta, C, s, workspace, thread_k=-1, thread_m=-1, sms=-1, max_p
         raise RuntimeError(f"k={prob_k} not compatible with {s.shape[0]} groups.")
     if workspace.numel() < prob_m // 128 * max_par:
         raise RuntimeError(f"workspace must be of size at least {prob_m // 128 * max_par}.")
-    if groupsize == -1 and prob_m % 128 == 0 and prob_k % 64 == 0:
+    if prob_m % 128 == 0 and prob_k % 64 == 0:
         _check_packed(B, meta, s, prob_m, prob_k)
     lib = _ffi.lib()
     split = lib.triteia_hip_bmm_scratch_bytes(prob_m, 1, prob_n, prob_k) if groupsize == -1 else 0

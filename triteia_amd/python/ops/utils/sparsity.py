@@ -133,6 +133,27 @@ def pack_2_4(q: torch.Tensor, lo: torch.Tensor, hi: torch.Tensor, scales: torch.
     return qweight, pack_meta(lo, hi), scales.reshape(1, m).to(torch.float16).contiguous()
 
 
+GROUP_K = 128   # dense k per scale group (groupsize 64 in the launchers' unit of compressed k)
+_GROUP_SCALE_ORDER = [i * 8 + j for i in range(8) for j in (0, 4, 1, 5, 2, 6, 3, 7)]
+
+
+def pack_group_scales(scales: torch.Tensor) -> torch.Tensor:
+    """Scales by (group of 128 dense k, column), [k/128, m] -> the tensor `mul_2_4` takes as `s`: every run of 64
+    columns in the reference's stored order (triteia/python/ops/utils/sparsity.py:54-57, nn/linear.py:117)."""
+    g, m = scales.shape
+    order = torch.tensor(_GROUP_SCALE_ORDER, device=scales.device)
+    return scales.to(torch.float16).reshape(-1, 64)[:, order].reshape(g, m).contiguous()
+
+
+def unpack_group_scales(stored: torch.Tensor) -> torch.Tensor:
+    """Inverse of `pack_group_scales`."""
+    g, m = stored.shape
+    order = torch.tensor(_GROUP_SCALE_ORDER, device=stored.device)
+    out = torch.empty((g * m // 64, 64), dtype=stored.dtype, device=stored.device)
+    out[:, order] = stored.reshape(-1, 64)
+    return out.reshape(g, m)
+
+
 def unpack_2_4(qweight: torch.Tensor, meta: torch.Tensor, scales: torch.Tensor = None, dtype=torch.float16):
     """Packed tensors -> dense [k, m] weight (x @ W convention).  With `scales` the result is
     fp16(q) * scale (rounded to fp16 like the reference's dequantised test weight,
@@ -147,4 +168,7 @@ def unpack_2_4(qweight: torch.Tensor, meta: torch.Tensor, scales: torch.Tensor =
     dense = dense.reshape(m, 2 * k2).t().contiguous()
     if scales is None:
         return dense.to(dtype)
+    if scales.dim() == 2 and scales.shape[0] > 1:      # grouped: stored scales per (128 dense k, column)
+        per_row = unpack_group_scales(scales.to(torch.float16)).repeat_interleave(GROUP_K, dim=0)
+        return (dense.to(torch.float16) * per_row).to(dtype)
     return (dense.to(torch.float16) * scales.reshape(1, m).to(torch.float16)).to(dtype)
