@@ -139,6 +139,14 @@ def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
     padded = ops.matmul_4bit_2_4(gq, gx, gm, gs)
     torch.cuda.synchronize()
     assert torch.equal(padded, out), "the order of the units changed bits"
+    # ... and from the padded order on, a block of column groups x a block of token tiles per XCD, in every block size
+    # that cuts this layer's padded column groups over the 8 XCDs (sizes that do not are ignored)
+    for block in (1, 2, 4, 8, 16):
+        setknob(monkeypatch, "TRITEIA_HIP_XCD_CGS", str(block))
+        blocks = ops.matmul_4bit_2_4(gq, gx, gm, gs)
+        torch.cuda.synchronize()
+        assert torch.equal(blocks, out), f"blocks of {block} column groups per XCD changed bits"
+    delknob(monkeypatch, "TRITEIA_HIP_XCD_CGS")
     delknob(monkeypatch, "TRITEIA_HIP_WIDE_ORDER_MIN_IDLE")
     setknob(monkeypatch, "TRITEIA_HIP_XCD_SWIZZLE", "2")
     unpadded = ops.matmul_4bit_2_4(gq, gx, gm, gs)
@@ -746,6 +754,14 @@ def test_plan_lists_64_token_tiles_for_wide_layers(ops, monkeypatch, T, N, k, m,
     sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
     torch.cuda.synchronize()
     assert torch.equal(out, outs["1"]), "the order of the units changed bits"
+    # blocks of column groups x blocks of tiles per XCD (the blocks of tiles are cut on the device from the plan's real
+    # number of tiles, the launch from the host's bound)
+    for block in (1, 2, 4, 8):
+        setknob(monkeypatch, "TRITEIA_HIP_XCD_CGS", str(block))
+        out = torch.full((T, m), -3.0, dtype=torch.float16, device=DEV)
+        sbmm_2_4_routed(gx, gq, gm, out, gs, gi)
+        torch.cuda.synchronize()
+        assert torch.equal(out, outs["1"]), f"blocks of {block} column groups per XCD changed bits"
 
 
 def test_empty_and_degenerate_inputs(ops, plan_rules):
