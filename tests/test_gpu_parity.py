@@ -616,6 +616,45 @@ def test_large_batches_through_the_plan(ops, T, N, k, m, seed, plan_rules):
     assert bool((out[torch.from_numpy(idx < 0).to(DEV)] == 0).all())
 
 
+@pytest.mark.parametrize("T,N,k,m,seed,hot", [
+    (600, 3, 256, 512, 111, False),      # a plan of 32-token tiles that also lists 64-token tiles: that list
+    (4000, 3, 256, 640, 112, False),     # a plan of 64-token tiles: its narrow-only list
+    (1500, 40, 256, 512, 113, True),     # many deltas with a few tokens each beside a hot one
+])
+def test_one_list_of_64_token_tiles_instead_of_the_split(ops, monkeypatch, T, N, k, m, seed, hot):
+    """A plan with wide tiles, on a layer whose wide launch is on: where one list of 64-token tiles over all tokens
+    needs no more rounds of workgroups than the wide tiles alone (on these small layers: always), the wide kernel takes
+    that list and the narrow kernel returns -- chosen on the device.  Against the oracle, and against the split
+    {wide tiles, narrow rest} (knob off), which adds over K in another order for the rest's rows."""
+    say(f"all-64 list T={T} N={N} k={k} m={m} seed={seed}")
+    from triteia_amd.python.capi import sbmm_2_4_routed
+    qw, meta, s = make_deltas(N, k, m, seed)
+    x = activations(T, k, seed + 1)
+    rng = np.random.default_rng(seed + 2)
+    idx = rng.integers(-1, N, size=T).astype(np.int32)
+    if hot:
+        idx[rng.random(T) < 0.5] = 1
+    ref = orc.sbmm_4bit_2_4(qw, x, meta, s, idx)
+    gq, gm, gs, gx, gi = to_gpu(qw, meta, s, x, idx)
+    setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", "1")
+    setknob(monkeypatch, "TRITEIA_HIP_MID", "0")
+    outs = {}
+    for all64 in ("1", "0"):
+        setknob(monkeypatch, "TRITEIA_HIP_PLAN_ALL64", all64)
+        for accumulate in (False, True):
+            out = torch.full((T, m), -3.0 if not accumulate else 0.5, dtype=torch.float16, device=DEV)
+            sbmm_2_4_routed(gx, gq, gm, out, gs, gi, accumulate=accumulate)
+            torch.cuda.synchronize()
+            outs[all64, accumulate] = out
+    none = torch.from_numpy(idx < 0).to(DEV)
+    for all64 in ("1", "0"):
+        assert bool((outs[all64, False][none] == -3.0).all()) and bool((outs[all64, True][none] == 0.5).all())
+        check_close(torch.where(none[:, None], torch.zeros_like(outs[all64, False]), outs[all64, False]), ref, what=f"all64={all64}")
+        check_close(torch.where(none[:, None], torch.zeros_like(outs[all64, True]), outs[all64, True] - 0.5), ref, tol=4e-3, what=f"all64={all64}, added")
+    rel = ((outs["1", False].float() - outs["0", False].float()).norm() / outs["0", False].float().norm()).item()
+    assert rel < 1e-3, rel
+
+
 @pytest.mark.parametrize("T,N,k,m,seed", [(64, 1, 512, 384, 95), (150, 2, 256, 640, 96), (100, 1, 320, 128, 97)])
 def test_few_deltas_take_their_tiles_in_split_passes(ops, monkeypatch, T, N, k, m, seed, plan_rules):
     """One or two deltas with tens of tokens on a narrow layer: the plan's 64-token tiles are taken in
@@ -664,6 +703,7 @@ def test_plan_tiles_on_the_32_token_wide_kernel(ops, monkeypatch, T, N, k, m, se
     say(f"32-token wide kernel T={T} N={N} k={k} m={m} seed={seed} wide_bar={wide_bar}")
     from triteia_amd.python.capi import sbmm_2_4_routed
     setknob(monkeypatch, "TRITEIA_HIP_FUSED_ROUTE", "0")
+    setknob(monkeypatch, "TRITEIA_HIP_PLAN_ALL64", "0")   # (with MID=0 the narrow kernel is to take its share of the plan)
     setknob(monkeypatch, "TRITEIA_HIP_PLAN_WIDE_MIN_UNITS", wide_bar)
     qw, meta, s = make_deltas(N, k, m, seed)
     x = activations(T, k, seed + 1)

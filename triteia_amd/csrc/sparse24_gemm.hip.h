@@ -116,7 +116,24 @@ struct Sparse24Args {
   // (workgroups 2g and 2g + 1 of a column group; a half without tokens returns at once)
   int tile_halves;
   int scale_groups;         // 0: one scale per output column; else k / 128 groups of K, each with a scale per column
+  // A plan with wide tiles on a layer whose wide launch fills the chip.  The wide kernel leaves a delta's last tokens
+  // (fewer than 64) to the narrow kernel, a second stream of that delta's weights.  Where ONE list of 64-token tiles
+  // over all tokens (tiles_all64; plan_header[all64_index] of them) needs no more rounds of the workgroups that run
+  // together than the wide tiles alone, the wide kernel takes that list and the narrow kernel returns at once: decided
+  // on the device, by both kernels alike, from the numbers of tiles in the plan's header.  nullptr: never.
+  const int4* tiles_all64;
+  const int* plan_header;
+  int all64_index;
 };
+
+// workgroups of the 64-token wide kernel that run together: two on each of 256 CUs
+constexpr int kWideSlots = 512;
+__device__ __forceinline__ bool plan_takes_all64(const Sparse24Args& p) {
+  const int wide = p.plan_header[4], all = p.plan_header[p.all64_index];
+  if ((long)wide * p.wide_gate < p.wide_min_units) return false;   // (no wide launch at all: the narrow kernel takes every token)
+  // wide_gate = column groups of the layer = workgroups per tile
+  return (all * p.wide_gate + kWideSlots - 1) / kWideSlots <= (wide * p.wide_gate + kWideSlots - 1) / kWideSlots;
+}
 
 __device__ __forceinline__ uint32_t h2_bits(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
 __device__ __forceinline__ half2_t bits_h2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -630,6 +647,8 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 && !GS ? 3 : 2) : (
       if ((long)p.n_groups_dev[4] * p.wide_gate < p.wide_min_units) {
         d = d_alt;
         alt_list = true;
+      } else if (p.tiles_all64 && plan_takes_all64(p)) {
+        return;   // the wide kernel takes every token of this plan
       }
     }
     delta = d.x;

@@ -109,8 +109,19 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
   }
   int delta, start, count;
   bool alt_list = false;
+  int all64_live = -1;
   if (p.tiles) {
-    int4 d = p.tiles[grp];
+    const int4* list = p.tiles;
+    if (!PLAN_ALL && p.tiles_all64) {
+      // the plan's wide tiles, or one list of 64-token tiles over all its tokens (the choice comes first: the launch
+      // is sized for the longer of the two lists, and a workgroup past the end of the chosen one reads no tile)
+      if (plan_takes_all64(p)) {
+        list = p.tiles_all64;
+        all64_live = p.plan_header[p.all64_index];
+      }
+      if (grp >= (all64_live >= 0 ? all64_live : p.n_groups_dev[0])) return;
+    }
+    int4 d = list[grp];
     if (PLAN_ALL && p.tiles_alt) {
       // this build stands in for the narrow kernel on a plan's narrow tiles: like that kernel it takes
       // the narrow-only list when the plan's wide tiles do not fill the chip (both candidates are requested together)
@@ -130,8 +141,8 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
     start = gi * p.uniform_stride + p.uniform_first + tc * TOK;
     count = min(TOK, p.uniform_count - tc * TOK);
   }
-  const int n_groups = p.n_groups_dev ? p.n_groups_dev[alt_list ? 5 : 0] : p.n_groups;
-  if (!PLAN_ALL && p.wide_min_units && (long)n_groups * p.wide_gate < p.wide_min_units) return;   // the narrow kernel has taken these tokens
+  const int n_groups = all64_live >= 0 ? all64_live : (p.n_groups_dev ? p.n_groups_dev[alt_list ? 5 : 0] : p.n_groups);
+  if (!PLAN_ALL && all64_live < 0 && p.wide_min_units && (long)n_groups * p.wide_gate < p.wide_min_units) return;   // the narrow kernel has taken these tokens
   if (grp >= n_groups) return;
   if (delta < 0 || delta >= p.n_deltas || count <= 0) return;
   const int cnt = min(count, TOK);

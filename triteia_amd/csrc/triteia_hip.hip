@@ -59,7 +59,7 @@ struct Knobs {
   int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, xcd_cgs = 0 /* 0: the rule, n > 0: blocks of n column groups, -1: never */, wide_order_min_idle = kUnset, pass_nt = 0;
   int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
-  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1, lora_mfma = 1;
+  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1, plan_all64 = 1, lora_mfma = 1;
   int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
   int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset, share16 = 1, share16_max_blocks = kUnset;
 };
@@ -75,7 +75,7 @@ void read_knobs() {
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
       {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
       {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
-      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"PLAN_BIG", &k.plan_big}, {"LORA_MFMA", &k.lora_mfma}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
+      {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"PLAN_BIG", &k.plan_big}, {"PLAN_ALL64", &k.plan_all64}, {"LORA_MFMA", &k.lora_mfma}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
       {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
       {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift}, {"SHARE16", &k.share16}, {"SHARE16_MAX_BLOCKS", &k.share16_max_blocks},
   };
@@ -1016,6 +1016,22 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     wide_launch = !mid && prob_k % 128 == 0 && (long)prob_n * prob_k * 2 < (1L << 32) &&
                   (long)(prob_n / 48 + 1) * a.wide_gate >= a.wide_min_units;
     if (!wide_launch) a.wide_min_units = 0x7fffffff;
+    // One list of 64-token tiles over all tokens, for the device to take instead of {wide tiles, narrow rest} where that
+    // costs no further round of workgroups (Sparse24Args::tiles_all64): the plan's narrow-only list when it is cut in
+    // 64-token tiles, else its list of 64-token tiles beside the 32-token ones, if it has one.  Measured by forcing that
+    // list on 16 deltas of 4096 x 4096: 2048 / 3072 tokens 77 -> 70, 92 -> 78 us, 8 deltas with 4096 tokens 98 -> 83 us
+    // (the same rounds either way), 16 / 32 deltas with 4096 tokens 102 -> 118, 119 -> 130 us (a further round: the
+    // split stays).
+    if (wide_launch && knobs().plan_all64) {
+      a.plan_header = ws + L.header;
+      if (tile == 64) {
+        a.tiles_all64 = reinterpret_cast<const int4*>(ws + L.all);
+        a.all64_index = 5;
+      } else if (plan_has_big(prob_n, n_deltas)) {
+        a.tiles_all64 = reinterpret_cast<const int4*>(ws + L.big);
+        a.all64_index = 6;
+      }
+    }
   }
   // The plan's tiles are cut without knowledge of the layer.  Where they make a launch of very few
   // workgroups on this layer (one or two deltas, a narrow matrix: fewer than 200 even on the plan's
@@ -1066,6 +1082,10 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
     a.tiles_alt = nullptr;
     a.n_groups_dev = ws + L.header + 4;
     a.n_groups = L.max_wide;
+    if (a.tiles_all64) {   // (the launch covers the longer of the two lists the device may choose from)
+      const int all64_max = a.all64_index == 5 ? plan_max_tiles(prob_n, n_deltas, 64) : L.max_big;
+      if (all64_max > a.n_groups) a.n_groups = all64_max;
+    }
     return launch_wide(a, static_cast<hipStream_t>(stream));
   }
   return TRITEIA_HIP_OK;
