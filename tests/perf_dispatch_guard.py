@@ -68,7 +68,7 @@ ROUTED_GRID = [
 # 64-token tiles for the wide kernel and rests for the K-split kernel keeps the launch within one round and is 15-19 %
 # ahead here; a host rule for it was measured and is a coin flip (the same split is 15-20 % behind with 8 deltas randomly
 # routed and 4-9 % behind evenly routed, 15 % ahead Zipf-routed): only the device knows whether a batch spills.
-KNOWN_GAPS = {(4096, 11008, 32, 512): 1.15, (8192, 8192, 16, 2048): 1.25}
+KNOWN_GAPS = {(4096, 11008, 32, 512): 1.15, (8192, 8192, 16, 2048): 1.30}
 # (k, m, tokens): single-matrix products around the windows of the wide kernels and of the K split
 UNIFORM_GRID = [
     (4096, 4096, 16), (4096, 4096, 128), (4096, 4096, 512), (4096, 4096, 640), (4096, 4096, 1024), (4096, 4096, 1536),

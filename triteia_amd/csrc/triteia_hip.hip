@@ -878,7 +878,14 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
     // as long as the launch has work for the chip (16 deltas with 512 tokens, 256 units on the bound: 45 -> 50 us) and
     // the batch is not one whose hot deltas fill the chip with 64-token tiles of their own (16 deltas, 4096 tokens:
     // 134 -> 153 us).
-    return knobs().mid_narrow && prob_n >= kMidNarrowMinTokens && prob_n < kMidNarrowMaxTokens && tiles * cgs >= (tile == 64 ? kMidNarrowMinUnits64 : kMidNarrowMinUnits);
+    // Past 2047 tokens the same holds for as long as the batch's 64-token tiles (tokens / 64 and half a tile per delta,
+    // as a randomly routed batch leaves them) fit one round of the 512 workgroups of the 64-token kernel that run
+    // together, with 48 tokens per delta and more (emptier tiles lose): 16 deltas with 2048 / 3072 tokens 77-80 -> 70-72,
+    // 92 -> 78 us, while with 4096 tokens (a third of a round too many) the split stays ahead, 102 against 118 us.
+    const long groups = n_deltas < prob_n ? n_deltas : prob_n;
+    const bool one_round = prob_n >= 48 * groups && (prob_n / 64 + (groups + 1) / 2) * cgs <= 512;
+    return knobs().mid_narrow && prob_n >= kMidNarrowMinTokens && (prob_n < kMidNarrowMaxTokens || one_round) &&
+           tiles * cgs >= (tile == 64 ? kMidNarrowMinUnits64 : kMidNarrowMinUnits);
   }
   return tiles * cgs >= knob_or(knobs().mid_min_units, kMidMinUnits);
 }
