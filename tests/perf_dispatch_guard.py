@@ -42,7 +42,7 @@ UNIFORM_ALTERNATIVES = {
     "32-token wide tiles, 8 wavefronts": {"TRITEIA_HIP_TILE256": "0", "TRITEIA_HIP_KSPLIT": "0", "TRITEIA_HIP_WIDE32_MIN_UNITS": "1", "TRITEIA_HIP_WIDE32_MAX_UNITS": BIG, "TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS": BIG, "TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS": "0"},
     "64-token wide tiles": {"TRITEIA_HIP_TILE256": "0", "TRITEIA_HIP_KSPLIT": "0", "TRITEIA_HIP_WIDE32_MAX_UNITS": "0", "TRITEIA_HIP_WIDE_MIN_UNITS": "1", "TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS": BIG, "TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS": "0"},
     "64-token wide tiles, 8 wavefronts": {"TRITEIA_HIP_TILE256": "0", "TRITEIA_HIP_KSPLIT": "0", "TRITEIA_HIP_WIDE32_MAX_UNITS": "0", "TRITEIA_HIP_WIDE_MIN_UNITS": "1", "TRITEIA_HIP_WIDE32_KSPLIT_MAX_UNITS": "0", "TRITEIA_HIP_WIDE64_KSPLIT_MAX_UNITS": BIG},
-    "256-token tiles": {"TRITEIA_HIP_TILE256_MIN_UNITS": "1", "TRITEIA_HIP_TILE256_MAX_UNITS": BIG, "TRITEIA_HIP_KSPLIT": "0"},
+    "256-token tiles": {"TRITEIA_HIP_TILE256": "2", "TRITEIA_HIP_TILE256_MIN_UNITS": "1", "TRITEIA_HIP_TILE256_MAX_UNITS": BIG, "TRITEIA_HIP_KSPLIT": "0"},
 }
 
 # (k, m, deltas, tokens): routed batches around the thresholds of in-kernel routing (64 / 256 tokens, 16 / 32 / 64

@@ -119,7 +119,7 @@ def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
     say(f"matmul {kernel} n={n} k={k} m={m} seed={seed}")
     setknob(monkeypatch, "TRITEIA_HIP_WIDE_MIN_UNITS", "1")
     setknob(monkeypatch, "TRITEIA_HIP_TILE256_MIN_UNITS", "1")
-    setknob(monkeypatch, "TRITEIA_HIP_TILE256", "1" if kernel == "tile256" else "0")
+    setknob(monkeypatch, "TRITEIA_HIP_TILE256", "2" if kernel == "tile256" else "0")   # (2: on layers of any width)
     if kernel in ("wide32", "wide32ks"):   # takes the tokens ahead of the other two whenever its window of units is open
         setknob(monkeypatch, "TRITEIA_HIP_WIDE32_MIN_UNITS", "1")
         setknob(monkeypatch, "TRITEIA_HIP_WIDE32_MAX_UNITS", "1000000000")
@@ -161,8 +161,11 @@ def test_matmul_wide_kernels(ops, monkeypatch, kernel, n, k, m, seed):
     assert rel < 1e-4, rel
 
 
-def test_matmul_many_tokens_reference_test_shape(ops):
-    # the reference's own test shape m = n = k = 4096 (tests/ops/test_matmul.py:30)
+@pytest.mark.parametrize("tile256", ["0", "2"])
+def test_matmul_many_tokens_reference_test_shape(ops, monkeypatch, tile256):
+    # the reference's own test shape m = n = k = 4096 (tests/ops/test_matmul.py:30): on the 64-token kernel, which the
+    # rules give it, and on the 256-token tile kernel, whose window of units it fills
+    setknob(monkeypatch, "TRITEIA_HIP_TILE256", tile256)
     n = k = m = 4096
     say(f"matmul n={n} k={k} m={m}")
     qw, meta, s = make_deltas(1, k, m, 77)

@@ -545,7 +545,12 @@ UniformPlan decide_uniform(int tokens, int stride, int n_groups, int m, int k, l
     }
   }
   // Groups of hundreds of tokens: 256-token x 256-column tiles whose wavefronts share the dequantised weights.
-  if (knobs().tile256 && wide_enabled() && x_below_4g) {
+  // On layers of fewer than 8 column groups of 512 (m < 3584) only: elsewhere the 64-token kernel, since its units go to
+  // the XCDs in blocks of column groups x token tiles, is as fast or faster inside this window (4096 x 4096 with 3072 /
+  // 3584 / 4096 tokens 80.5 -> 66.8, 80.7 -> 72.4, 81.7 -> 78.2 us; 4096 x 8192 with 2048 tokens 81.5 -> 78.8; 8192 x 4096
+  // and 11008 x 4096 with 4096 tokens 147.3 -> 145, 193 -> 192 us), while 4096 x 2048 with 8192 tokens, whose four column
+  // groups leave half of a padded tile's slots idle, keeps it (81 against 85 us).  The knob tile256 = 2 lifts the limit.
+  if (knobs().tile256 && (cgs < 8 || knobs().tile256 > 1) && wide_enabled() && x_below_4g) {
     const long ncp = (m / 128 + 1) / 2;
     const long min_units = knob_or(knobs().tile256_min_units, kTile256MinUnits);
     int t = tokens / kT256Tokens * kT256Tokens;
