@@ -132,7 +132,8 @@ def test_dispatch_queries_at_the_documented_points():
     assert lib.triteia_hip_bmm_scratch_bytes(4096, 1, 16, 4096) == 0
     assert uniform(4096, 1, 1024, 4096, 1) == 33       # 32-token tiles on eight wavefronts (one workgroup per CU)
     assert uniform(4096, 1, 1536, 4096, 1) == 65       # 64-token tiles on eight wavefronts
-    assert uniform(4096, 1, 4096, 4096, 1) == 256      # one round of 256-token tiles
+    assert uniform(4096, 1, 4096, 4096, 1) == 64       # 64-token tiles, two workgroups per CU
+    assert uniform(2048, 1, 8192, 4096, 1) == 256      # a narrow layer: one round of 256-token tiles
     assert uniform(28672, 1, 4096, 8192, 1) == 64      # several rounds: 64-token tiles, two workgroups per CU
     assert uniform(4096, 1, 128, 4096, 1) == 0
     assert uniform(100, 1, 16, 4096, 1) == -1          # not a legal shape
