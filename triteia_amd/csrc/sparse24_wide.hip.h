@@ -88,7 +88,9 @@ __global__ __launch_bounds__(256 * KS, KS == 1 ? 2 : 1) void sparse24_wide_kerne
     int rows_live = rows_of_tiles;
     if (p.tiles && p.n_groups_dev) {
       const bool alt = PLAN_ALL && p.tiles_alt && (long)p.n_groups_dev[4] * p.wide_gate < p.wide_min_units;
-      rows_live = min(rows_of_tiles, p.n_groups_dev[alt ? 5 : 0] * (PLAN_ALL && TOK == 32 && p.tile_halves ? 2 : 1));
+      int live = p.n_groups_dev[alt ? 5 : 0];
+      if (!PLAN_ALL && p.tiles_all64 && plan_takes_all64(p)) live = p.plan_header[p.all64_index];   // (the list chosen below)
+      rows_live = min(rows_of_tiles, live * (PLAN_ALL && TOK == 32 && p.tile_halves ? 2 : 1));
     }
     const int n_cgb = cg_pad / p.xcd_cgs;             // blocks of column groups (a divisor of 8)
     const int tbs = 8 / n_cgb;                         // blocks of tiles

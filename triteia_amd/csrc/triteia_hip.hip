@@ -389,7 +389,8 @@ static unsigned plan_wide_grid(Sparse24Args& b, long rows, int m, int tok, int p
   }
   return (unsigned)wide_grid_units(rows, m, b.xcd_swizzle);
 }
-int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
+// (`plan_tokens`, `plan_deltas`: the batch behind a plan's list of tiles, for the order of its units; 0 for uniform groups)
+int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens, int plan_tokens = 0, int plan_deltas = 0) {
   if (a.n_groups <= 0 || a.m == 0 || a.k == 0) return TRITEIA_HIP_OK;
   const long cgs = (a.m / 128 + 3) / 4;
   const long cg_pad = (cgs + 7) / 8 * 8;
@@ -399,7 +400,8 @@ int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens) {
   Sparse24Args b = a;
   if (!b.tiles) b.n_groups = (int)(a.n_groups * chunks);
   b.xcd_swizzle = wide_unit_order(a.m);
-  unsigned grid = (unsigned)wide_grid_units((long)a.n_groups * chunks, a.m, b.xcd_swizzle);
+  unsigned grid = a.tiles && plan_tokens > 0 ? plan_wide_grid(b, (long)a.n_groups * chunks, a.m, tok, plan_tokens, plan_deltas, 64)
+                                             : (unsigned)wide_grid_units((long)a.n_groups * chunks, a.m, b.xcd_swizzle);
   // Uniform launches: an XCD takes a block of column groups x a block of token tiles (order 4) where that makes its
   // L2 fetch fewer bytes than a run of column groups for every tile (order 1).  While the workgroups that an XCD holds at
   // a time (32 CUs x 1 or 2) walk K, its L2 fetches the packed weights of their distinct column groups and the
@@ -1098,7 +1100,7 @@ int triteia_hip_sbmm_2_4_planned(const void* A, const void* B, const void* meta,
       const int all64_max = a.all64_index == 5 ? plan_max_tiles(prob_n, n_deltas, 64) : L.max_big;
       if (all64_max > a.n_groups) a.n_groups = all64_max;
     }
-    return launch_wide(a, static_cast<hipStream_t>(stream));
+    return launch_wide(a, static_cast<hipStream_t>(stream), kWideTokens, prob_n, n_deltas);
   }
   return TRITEIA_HIP_OK;
 }
