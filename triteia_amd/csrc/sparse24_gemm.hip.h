@@ -99,7 +99,7 @@ struct Sparse24Args {
   int accumulate;           // 0: out = result, 1: out += result
   int raw_static;           // fused routing with group g = delta g: weights are requested before the indices arrive
   int rot_spread;           // steps between the starting points of consecutive deltas' walks over K (0: all start at step 0)
-  int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run
+  int xcd_swizzle;          // 1: remap column blocks so that each XCD owns a contiguous run; 5 (streaming kernel): whole groups per XCD
   int xcd_cgs;              // wide kernel, order 4: column groups (of 512) in the block that one XCD takes
   // K split across workgroups (uniform groups only): blockIdx.z = z takes the steps [z * ksplit_steps, (z + 1) * ksplit_steps)
   // of K and writes its fp32 sums, unscaled, to partial[z][row][column]; splitk_reduce_kernel adds the splits in
@@ -512,9 +512,20 @@ __global__ __launch_bounds__(64 * KW, (NT == 1 ? (DEPTH == 1 && !GS ? 3 : 2) : (
   const int col_units = (p.m >> 7) << p.sub_shift;
   const int cu_pad = (col_units + 7) & ~7;
   const int unit = blockIdx.x;
-  const int grp = unit / cu_pad;
-  const int i = unit - grp * cu_pad;
-  const int cu = p.xcd_swizzle ? (i & 7) * (cu_pad >> 3) + (i >> 3) : i;
+  int grp = unit / cu_pad;
+  int i = unit - grp * cu_pad;
+  int cu = p.xcd_swizzle ? (i & 7) * (cu_pad >> 3) + (i >> 3) : i;
+  if (p.xcd_swizzle == 5) {
+    // Whole groups per XCD, for launches whose groups all have work (the host asks for this order only then): the
+    // first 8 * gpx groups go gpx to an XCD, with all their column units, so that an XCD's L2 fetches the activations
+    // of its own groups only and streams whole matrices; the groups that are left over keep the order above.
+    const int gpx = p.n_groups >> 3;
+    if (unit < 8 * gpx * cu_pad) {
+      const int xcd = unit & 7, s = unit >> 3;
+      grp = xcd * gpx + s / cu_pad;
+      cu = s - (s / cu_pad) * cu_pad;
+    }
+  }
   if (cu >= col_units) return;
   const int cb = cu >> p.sub_shift;
 

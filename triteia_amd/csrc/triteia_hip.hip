@@ -245,6 +245,18 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
   }
   const long units = (long)a.n_groups * cb_pad;
   if (units > 0x7fffffffL) return fail(TRITEIA_HIP_ERR_PROB_SHAPE, "too many work units (%ld)", units);
+  // Launches whose groups all have work -- uniform groups, and a batch routed in the kernel with a group per delta --
+  // give whole groups to an XCD (Sparse24Args::xcd_swizzle = 5) instead of a run of column blocks of every group:
+  // each XCD's L2 then fetches the activations and indices of its own groups only (the counters showed them fetched once
+  // per XCD: 5.6 % on top of the algorithmic bytes of the 64-token batch over 16 deltas of 4096 x 4096) and streams whole
+  // matrices.  Measured: that batch 22.9 -> 22.3 us (four pairs of runs, each ahead); 8 matrices of 4096 x 4096 with a token
+  // each 13.9 -> 13.7 us; 12 deltas with 64 tokens 20.5 -> 20.2 us.  The sums do not depend on which workgroup takes which unit.
+  // Only for launches of a single round (at most the 512 workgroups that run together): there every XCD's share is
+  // resident at once whatever its size, while a longer launch needs the even split of every group over the XCDs
+  // (8 matrices of 4096 x 11008 with a token each, 704 workgroups: 30.4 -> 31.1 us; 16 deltas of 4096 x 11008 with 128
+  // tokens 63.0 -> 64.8 us).
+  if (a.xcd_swizzle == 1 && a.n_groups >= 8 && units * tsplit * zsplit <= 512 && (uniform || (a.raw_indices && a.raw_static))) a.xcd_swizzle = 5;
+  else if (a.xcd_swizzle == 5) a.xcd_swizzle = 1;
   const dim3 grid((unsigned)units, (unsigned)tsplit, (unsigned)zsplit);
 #define TRY(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
 #define TRY_EAGER(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_, true>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
