@@ -106,3 +106,35 @@ def test_the_idle_slots_balance_the_xcds():
             loads[order] = load
         assert max(loads[3]) < max(loads[1]), (cgs, rows, loads)
         assert lib.triteia_hip_wide_unit_order(512 * cgs) == (3 if (cgs + 7) // 8 * 8 - cgs >= 3 else 1)
+
+
+def streaming_unit_of(u, n_groups, col_units, order):
+    """(group, column unit) of workgroup u of sparse24_grouped_kernel, or None for a padding slot (the kernel's first
+    lines, restated): order 1 gives every XCD (u % 8) a run of column units of every group, order 5 whole groups."""
+    cu_pad = (col_units + 7) // 8 * 8
+    grp, i = divmod(u, cu_pad)
+    cu = (i & 7) * (cu_pad >> 3) + (i >> 3)
+    if order == 5:
+        gpx = n_groups >> 3
+        if u < 8 * gpx * cu_pad:
+            xcd, s = u & 7, u >> 3
+            grp, cu = xcd * gpx + s // cu_pad, s % cu_pad
+    return (grp, cu) if cu < col_units else None
+
+
+def test_whole_groups_per_xcd_in_the_streaming_kernel():
+    for n_groups in range(8, 41):
+        for col_units in (1, 2, 7, 8, 32, 43, 86, 224):
+            cu_pad = (col_units + 7) // 8 * 8
+            seen = collections.Counter()
+            groups_of_xcd = collections.defaultdict(set)
+            for u in range(n_groups * cu_pad):
+                t = streaming_unit_of(u, n_groups, col_units, 5)
+                if t is not None:
+                    seen[t] += 1
+                    if t[0] < (n_groups >> 3) * 8:
+                        groups_of_xcd[u % 8].add(t[0])
+            assert len(seen) == n_groups * col_units and set(seen.values()) == {1}, (n_groups, col_units)
+            # the groups that fill the XCDs evenly go whole to one XCD each, n_groups // 8 per XCD
+            assert all(len(v) == n_groups >> 3 for v in groups_of_xcd.values())
+            assert len(set().union(*groups_of_xcd.values())) == (n_groups >> 3) * 8
