@@ -56,11 +56,11 @@ int check_launch(const char* what) {
 // kUnset marks knobs whose default depends on the launch.
 constexpr int kUnset = -0x7fffffff;
 struct Knobs {
-  int nt = 0, kw = kUnset, depth = kUnset, rot_spread = kUnset, xcd_swizzle = 1, xcd_cgs = 0 /* 0: the rule, n > 0: blocks of n column groups, -1: never */, wide_order_min_idle = kUnset, pass_nt = 0;
-  int wide = 1, wide_depth = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
+  int nt = 0, xcd_swizzle = 1, xcd_cgs = 0 /* 0: the rule, n > 0: blocks of n column groups, -1: never */, wide_order_min_idle = kUnset, pass_nt = 0;
+  int wide = 1, wide_min_units = kUnset, wide_min_batch = 256, plan_wide_min_units = kUnset;
   int wide32_min_units = kUnset, wide32_max_units = kUnset, wide32_ksplit_max_units = kUnset, wide64_ksplit_max_units = kUnset;
-  int mid = 1, mid64 = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1, plan_all64 = 1, lora_mfma = 1;
-  int eager = 1, fused_route = 1, fused_max_tokens = kUnset;
+  int mid = 1, mid64_max_k = 0x7fffffff, mid_min_column_groups = 16, mid_min_units = kUnset, mid_min_half_tokens = 7, mid_narrow = 1, mid_depth = 0, plan_big = 1, plan_all64 = 1, lora_mfma = 1;
+  int eager = 1, fused_route = 1;
   int tile256 = 1, tile256_min_units = kUnset, tile256_max_units = kUnset, ksplit = 1, sub_shift = kUnset, share16 = 1, share16_max_blocks = kUnset;
 };
 Knobs g_knobs;
@@ -69,14 +69,14 @@ std::once_flag g_knobs_once;
 void read_knobs() {
   Knobs k;
   struct { const char* name; int* dst; } table[] = {
-      {"NT", &k.nt}, {"KW", &k.kw}, {"DEPTH", &k.depth}, {"ROT_SPREAD", &k.rot_spread}, {"XCD_SWIZZLE", &k.xcd_swizzle}, {"XCD_CGS", &k.xcd_cgs}, {"WIDE_ORDER_MIN_IDLE", &k.wide_order_min_idle},
-      {"PASS_NT", &k.pass_nt}, {"WIDE", &k.wide}, {"WIDE_DEPTH", &k.wide_depth}, {"WIDE_MIN_UNITS", &k.wide_min_units},
+      {"NT", &k.nt}, {"XCD_SWIZZLE", &k.xcd_swizzle}, {"XCD_CGS", &k.xcd_cgs}, {"WIDE_ORDER_MIN_IDLE", &k.wide_order_min_idle},
+      {"PASS_NT", &k.pass_nt}, {"WIDE", &k.wide}, {"WIDE_MIN_UNITS", &k.wide_min_units},
       {"WIDE_MIN_BATCH", &k.wide_min_batch}, {"PLAN_WIDE_MIN_UNITS", &k.plan_wide_min_units},
       {"WIDE32_MIN_UNITS", &k.wide32_min_units}, {"WIDE32_MAX_UNITS", &k.wide32_max_units},
       {"WIDE32_KSPLIT_MAX_UNITS", &k.wide32_ksplit_max_units}, {"WIDE64_KSPLIT_MAX_UNITS", &k.wide64_ksplit_max_units},
-      {"MID", &k.mid}, {"MID64", &k.mid64}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
+      {"MID", &k.mid}, {"MID64_MAX_K", &k.mid64_max_k}, {"MID_MIN_COLUMN_GROUPS", &k.mid_min_column_groups},
       {"MID_MIN_UNITS", &k.mid_min_units}, {"MID_MIN_HALF_TOKENS", &k.mid_min_half_tokens}, {"MID_NARROW", &k.mid_narrow}, {"MID_DEPTH", &k.mid_depth}, {"PLAN_BIG", &k.plan_big}, {"PLAN_ALL64", &k.plan_all64}, {"LORA_MFMA", &k.lora_mfma}, {"EAGER", &k.eager}, {"FUSED_ROUTE", &k.fused_route},
-      {"FUSED_MAX_TOKENS", &k.fused_max_tokens}, {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
+      {"TILE256", &k.tile256}, {"TILE256_MIN_UNITS", &k.tile256_min_units}, {"TILE256_MAX_UNITS", &k.tile256_max_units},
       {"KSPLIT", &k.ksplit}, {"SUB_SHIFT", &k.sub_shift}, {"SHARE16", &k.share16}, {"SHARE16_MAX_BLOCKS", &k.share16_max_blocks},
   };
   char name[64];
@@ -155,8 +155,7 @@ void launch_one(const Sparse24Args& a, dim3 grid, hipStream_t st) {
 // order as the eight-wavefront streaming kernel that took them before.  Returns the 16-column tiles per share, 0 = no.
 constexpr long kShare16MaxBlocks = 128;
 static int share16_tiles(long n_groups, int m, int tokens_per_group) {
-  if (tokens_per_group > 16 || !knobs().share16 || knobs().sub_shift != kUnset || knobs().kw != kUnset ||
-      knobs().depth != kUnset || knobs().nt != 0)
+  if (tokens_per_group > 16 || !knobs().share16 || knobs().sub_shift != kUnset || knobs().nt != 0)
     return 0;
   const long blocks = n_groups * (m / 128);
   if (blocks > knob_or(knobs().share16_max_blocks, kShare16MaxBlocks)) return 0;
@@ -188,7 +187,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
   // Only for uniform groups (matmul, bmm): the split of K among the wavefronts fixes the order of the
   // fp32 sums, and a routed token must have the same bits whatever the size of its batch.
   const bool one_per_cu = uniform && zsplit == 1 && (nt == 1 || nt == 2) && (long)a.n_groups * cb_pad * tsplit <= 256;
-  const int kw = knob_or(knobs().kw, one_per_cu ? 8 : 4);
+  const int kw = one_per_cu ? 8 : 4;
   // register budget: the 16-token kernel runs 3 workgroups per CU with one step in flight (2 with
   // two), the 32-token kernel 2 per CU with two, the 64-token kernel 1 per CU with one.  Fused
   // routing in its eager form keeps one step in flight (measured: a second step requested ahead of
@@ -209,11 +208,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
     if (live_groups > a.n_groups) live_groups = a.n_groups;
   }
   const bool small = live_groups * cb_pad * tsplit * zsplit <= 256.5;
-  const int depth = knob_or(knobs().depth, eager || kw == 8 ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1));
-  if (eager && !(kw == 4 && ((nt == 1 && depth == 2) || (nt == 1 && depth == 1) || (nt == 2 && depth == 1) || (nt == 4 && depth == 1)))) {
-    a.raw_static = 0;   // no eager build of this variant: route first, then request
-    a.n_groups = a.raw_count < a.n_deltas ? a.raw_count : a.n_deltas;
-  }
+  const int depth = eager || kw == 8 ? 1 : (nt == 2 || (nt == 1 && small) ? 2 : 1);
   // About 512 workgroups run at a time.  When those belong to four or more deltas (narrow matrices),
   // the deltas start their walks over K spread evenly around the ring of steps; wide matrices are
   // streamed one or two at a time anyway and walk from step 0.
@@ -223,7 +218,7 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
     const long side_by_side = 512 / (((long)(a.m / 128) + 7) / 8 * 8);
     const int n_steps = (a.k / 32 + 3) / 4;
     const long spread = side_by_side >= 4 ? n_steps / (side_by_side < 16 ? side_by_side : 16) : 0;
-    a.rot_spread = knob_or(knobs().rot_spread, spread);
+    a.rot_spread = (int)spread;
   }
   if (const int tiles = uniform && nt == 1 && tsplit == 1 && zsplit == 1 && !a.ksplit_steps ? share16_tiles(a.n_groups, a.m, a.uniform_count) : 0) {
     const long sh_pad = ((long)(a.m / (16 * tiles)) + 7) / 8 * 8;
@@ -261,10 +256,10 @@ int launch_sparse24(Sparse24Args a, int nt, long tsplit, hipStream_t st, int zsp
 #define TRY(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
 #define TRY_EAGER(NT_, KW_, D_) if (nt == NT_ && kw == KW_ && depth == D_) { launch_one<NT_, KW_, D_, true>(a, grid, st); return check_launch("sparse24_grouped_kernel"); }
   if (a.raw_indices && a.raw_static) {
-    TRY_EAGER(1, 4, 1) TRY_EAGER(1, 4, 2) TRY_EAGER(2, 4, 1) TRY_EAGER(4, 4, 1)
+    TRY_EAGER(1, 4, 1) TRY_EAGER(2, 4, 1) TRY_EAGER(4, 4, 1)
   }
-  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 4, 3) TRY(1, 8, 1) TRY(1, 8, 2)
-  TRY(2, 4, 1) TRY(2, 4, 2) TRY(2, 8, 1)
+  TRY(1, 4, 1) TRY(1, 4, 2) TRY(1, 8, 1)
+  TRY(2, 4, 2) TRY(2, 8, 1)
   TRY(4, 4, 1)
 #undef TRY
 #undef TRY_EAGER
@@ -459,10 +454,8 @@ int launch_wide(const Sparse24Args& a, hipStream_t st, int tok = kWideTokens, in
   else if (units <= knob_or(knobs().wide64_ksplit_max_units, kWide64KSplitMaxUnits) &&
            !a.tiles)   // (a plan's launch is sized by an upper bound on its tiles; at 190-230 real units it measured the same either way)
     hipLaunchKernelGGL((sparse24_wide_kernel<1, kWideTokens, false, 2>), dim3(grid), dim3(512), 0, st, b);
-  else if (knobs().wide_depth == 1)
-    hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3(grid), dim3(256), 0, st, b);
   else
-    hipLaunchKernelGGL((sparse24_wide_kernel<2>), dim3(grid), dim3(256), 0, st, b);
+    hipLaunchKernelGGL((sparse24_wide_kernel<1>), dim3(grid), dim3(256), 0, st, b);
   return check_launch("sparse24_wide_kernel");
 }
 
@@ -875,7 +868,7 @@ static bool mid_tiles(int prob_n, int n_deltas, int prob_m, int prob_k) {
   // with 2048 / 4096 tokens over 64 deltas 1454 -> 1317 / 1920 -> 1736 us, 2048 tokens over 32 deltas 985 -> 864 us;
   // 8192 x 8192 with 4096 tokens over 64 deltas 408 -> 381 us; k = 11008 .. 28672: 0-3 % faster.  The knob mid64_max_k
   // can cap it: before the wide kernel's loop lost its conditional waits, k >= 8192 was better off on the narrow kernel.)
-  const bool mid64 = tile == 64 && knobs().mid64 && prob_k < knobs().mid64_max_k;
+  const bool mid64 = tile == 64 && prob_k < knobs().mid64_max_k;
   if (!knobs().mid || (tile != 32 && !mid64)) return false;
   if (prob_k % 128 != 0 || (long)prob_n * prob_k * 2 >= (1L << 32)) return false;   // whole K steps, 32-bit activation offsets
   const long tiles = (n_deltas < prob_n ? n_deltas : prob_n) + prob_n / tile;
@@ -923,7 +916,7 @@ static bool routed_in_kernel(int prob_n, int n_deltas, int prob_m, int prob_k) {
   // 256 over at most 32 -- whatever the rules below say; for measurements)
   if (knobs().fused_route == 2) return prob_n <= kFusedMaxTokens && n_deltas <= (prob_n > 64 ? 32 : 64);
   if (prob_n > 32 && !routed_eager_ok(prob_n, n_deltas) && (long)prob_k * prob_m >= (1L << 25)) return false;
-  return prob_n <= knob_or(knobs().fused_max_tokens, kFusedMaxTokens) && prob_n <= kFusedMaxTokens &&
+  return prob_n <= kFusedMaxTokens &&
          n_deltas <= (prob_n > 64 ? 16 : 64) && knobs().fused_route &&
          !(prob_n >= 128 && ((!routed_eager_ok(prob_n, n_deltas) && mid_tiles(prob_n, n_deltas, prob_m, prob_k)) ||
                              (long)prob_k * prob_m >= (1L << 27)));
@@ -1364,6 +1357,7 @@ int sgmv_routed_impl(void* y, long y_stride, const void* x, long x_stride, const
   a.accumulate = accumulate;
   return launch_sgmv(a, prob_n, static_cast<hipStream_t>(stream), prob_n / (n_adapters < prob_n ? n_adapters : prob_n));
 }
+
 }  // namespace
 
 extern "C" {
