@@ -849,10 +849,18 @@ constexpr int kMidNarrowMinUnits = 280, kMidNarrowMinUnits64 = 150, kMidNarrowMi
 // gain is 4-10 % (16 deltas of 4096 x 4096 with 768 / 1024 tokens 49.6 -> 45.0, 57.0 -> 54.7 us).  Past two workgroups
 // per CU the third workgroup of the one-deep build is worth more (16 deltas of 4096 x 4096 with 2048 randomly routed
 // tokens, 640 units on the bound: 76.2 -> 84.8 us; 4 / 8 of 4096 x 11008 with 768 tokens 66.5 -> 77.4, 73.6 -> 83.6 us), so
-// the bound itself must fit; below 288 units the K-split narrow kernel is faster (16 deltas of 4096 x 4096 with 512
-// tokens 33.3 against 40.5 us), and so it is with few tokens per tile (256 tokens, Zipf(1.2) over 32 deltas of
-// 11008 x 4096, 6.4 per tile on the bound: 89.6 against 102.6 us).
-constexpr long kMidDeepMinUnits = 288, kMidDeepMaxUnits = 512, kMidDeepMinTokensPerTile = 12;
+// the bound itself must fit; below 240 units the K-split narrow kernel is faster (16 deltas of 4096 x 4096 with 320 / 384
+// randomly routed tokens, 208 / 224 units: 29.0 against 34.5, 31.4 against 34.6 us), and so it is with few tokens per tile
+// (256 tokens, Zipf(1.2) over 32 deltas of 11008 x 4096, 6.4 per tile on the bound: 89.6 against 102.6 us).
+// The lower end was 288 before the requests of this build moved in between its groups of MFMAs: its time is now flat
+// in the tokens up to a launch of one round (34 us on k = 4096, 57 on 8192, 74 on 11008), while the narrow kernel pays
+// a second round of workgroups from about 240 units on.  Randomly routed, narrow kernel -> this build: 16 deltas of
+// 4096 x 4096 with 448 / 512 tokens 37.9 -> 34.9, 42.0 -> 38.6 us, 8 with 704 45.0 -> 37.2, 20 with 384 38.5 -> 34.9; 4 of
+// 4096 x 11008 with 192 / 224 36.0 -> 33.2, 42.6 -> 33.3, 2 with 288 46.5 -> 32.5; 16 of 11008 x 4096 with 448 / 512 84 -> 74,
+// 90 -> 73.6; 8 / 4 of 8192 x 8192 with 288 / 352 / 416 62 -> 57.5, 68 -> 56.6, 69 -> 57.3; 2 of 8192 x 28672 with 96 65.5 -> 58.6 us.
+// It loses where the bound is far above the real tiles: 2 of 4096 x 11008 with 256 tokens a third of them unrouted
+// 31.0 -> 32.6, 8 of 8192 x 8192 with 224 54.0 -> 57.8, one 8192 x 28672 with 128 tokens half of them unrouted 50.0 -> 55.8 us.
+constexpr long kMidDeepMinUnits = 240, kMidDeepMaxUnits = 512, kMidDeepMinTokensPerTile = 12;
 static long mid_units32(int prob_n, int n_deltas, int prob_m, int tile) {
   const long cgs = (prob_m / 128 + 3) / 4, cg_pad = (cgs + 7) / 8 * 8;
   return (long)plan_max_tiles(prob_n, n_deltas, tile) * (tile == 64 ? 2 : 1) * cg_pad;
