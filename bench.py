@@ -528,6 +528,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    from triteia_amd import build as _build
+    _build.ensure_built(verbose=False)   # loads what is built in the tree; compiles only if there is nothing
     ffi.lib()   # fails loudly if the HIP library is missing
 
     shape = tuple(int(v) for v in a.shape.split(",")) if a.shape else None

@@ -30,6 +30,14 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+@pytest.fixture(scope="session", autouse=True)
+def _library_is_built():
+    """The tests load the library that is built in the tree and compile it only if there is none
+    (hipcc cross-compiles without a GPU)."""
+    from triteia_amd import build as _build
+    _build.ensure_built(verbose=False)
+
+
 @pytest.fixture(autouse=True)
 def _library_knobs_follow_environment():
     """Tests change TRITEIA_HIP_* variables through `monkeypatch`; the library snapshots them, so it is told to

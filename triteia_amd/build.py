@@ -58,5 +58,13 @@ def build(verbose: bool = True, extra_flags=()) -> str:
     return LIB
 
 
+def ensure_built(verbose: bool = True) -> str:
+    """The built library's path; compiles it first if (and only if) there is none in the tree.  For tests,
+    smoke runs and benchmarks, which load what is built; `build()` itself compiles every time."""
+    if not os.path.exists(LIB):
+        build(verbose=verbose)
+    return LIB
+
+
 if __name__ == "__main__":
     print(build(extra_flags=sys.argv[1:]))
